@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Headline benchmark: paged decode, Llama-7B layer shape, batch 64.
+
+One step = one pass of the decode hot path over one batch for one transformer
+layer: KV append of the 64 new K/V rows, then paged attention of the 64 query
+tokens against the block KV cache (32 q heads, 32 kv heads, head_dim 128,
+bf16, block 16, context lengths uniform in [512, 4096], randomly permuted
+block tables, q/K/V ~ N(0,1)).  Several layers' pools are resident and the
+steps rotate over them, as a decoder's layers do, so no step re-reads the
+bytes the previous one left in cache.
+
+Prints ONE JSON line.  `value` is achieved HBM GB/s of the whole step
+(algorithmic bytes / wall time per step); decode tokens/s are reported beside
+it.  `roofline` describes the decode call (main kernel + its split-K reduce)
+timed with events on the launch stream; `cpu_baseline` is the CPU oracle (the
+reference's dense attention arithmetic driven through the block table) timed
+on the host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, vendor figure
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=4, help="resident layer pools the steps rotate over")
+    ap.add_argument("--part-tokens", type=int, default=0, help="split-K partition size (0 = library default)")
+    ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the paged-attention path is single-GPU "
+                 "(sequences and KV heads shard without communication); run with --gpus 1")
+    import torch
+    from ironcore_amd import paged_ops, workloads
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the paged path has no CPU implementation)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    make = {"llama7b": workloads.llama7b_decode, "llama70b": workloads.llama70b_gqa_decode,
+            "grpo": workloads.qwen7b_grpo_decode}[args.workload]
+    wl = make(device=dev, seed=args.seed)
+    b, hn, gn, hd, bs = wl.batch, wl.hn, wl.gn, wl.hd, wl.block_size
+    # one pool pair per resident layer (layer 0 is the workload's own)
+    pools = [(wl.k_pool, wl.v_pool)]
+    for layer in range(1, args.layers):
+        g = torch.Generator(device=dev)
+        g.manual_seed(args.seed + 100 + layer)
+        pools.append(tuple(torch.randn(wl.k_pool.shape, generator=g, device=dev, dtype=torch.float32)
+                           .to(wl.k_pool.dtype) for _ in range(2)))
+    # the step's new K/V rows go to the slot of each sequence's last token
+    ctx = wl.context_lens.long()
+    last = ctx - 1
+    slot_mapping = (wl.block_tables.long().gather(1, (last // bs).unsqueeze(1)).squeeze(1) * bs + last % bs)
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed + 7)
+    k_new = torch.randn(b, gn, hd, generator=g, device=dev, dtype=torch.float32).to(wl.k_pool.dtype)
+    v_new = torch.randn(b, gn, hd, generator=g, device=dev, dtype=torch.float32).to(wl.k_pool.dtype)
+    out = torch.empty(b, hn * hd, dtype=wl.query.dtype, device=dev)
+
+    def step(i):
+        kp, vp = pools[i % len(pools)]
+        paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
+        paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
+                               wl.max_context_len, out=out, part_tokens=args.part_tokens)
+
+    # ---- parity gate on the tensors that are about to be timed --------------
+    from oracle import paged as oracle_paged
+    step(0)
+    torch.cuda.synchronize()
+    n_chk = min(b, 6)
+    ref = oracle_paged.paged_decode(wl.query[:n_chk].cpu(), pools[0][0].cpu(), pools[0][1].cpu(),
+                                    wl.block_tables[:n_chk].cpu(), wl.context_lens[:n_chk].cpu())
+    parity = (out[:n_chk].float().cpu() - ref.float()).abs().max().item()
+    if not parity <= 2e-2:
+        sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
+
+    # ---- timed region ---------------------------------------------------------
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        kp, vp = pools[i % len(pools)]
+        paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
+        ev[i][0].record()
+        paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
+                               wl.max_context_len, out=out, part_tokens=args.part_tokens)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    decode_ms = [a.elapsed_time(c) for a, c in ev]
+    decode_ms_avg = sum(decode_ms) / len(decode_ms)
+
+    es = wl.query.element_size()
+    decode_bytes = wl.algorithmic_bytes()
+    append_bytes = 2 * (2 * b * gn * hd * es) + 8 * b
+    step_bytes = decode_bytes + append_bytes
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = decode_bytes / (decode_ms_avg * 1e-3) / 1e9
+
+    result = {
+        "metric": "paged_decode_hbm_gbps",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "decode_tokens_per_s_per_layer": round(b / (ms_per_step * 1e-3), 1),
+        "decode_tokens_per_s_32_layers": round(b / (32 * ms_per_step * 1e-3), 1),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": wl.name, "batch": b, "q_heads": hn, "kv_heads": gn, "head_dim": hd,
+                   "block_size": bs, "sum_context": wl.logical_tokens, "unique_tokens": wl.unique_tokens,
+                   "resident_layers": len(pools), "part_tokens": args.part_tokens or 512,
+                   "step": "kv_append(64 rows) + paged_decode, one layer"},
+        "parity_max_abs_vs_oracle": parity,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "paged_decode_kernel (+ split-K reduce)",
+                     "bytes_per_launch": decode_bytes, "avg_launch_ms": round(decode_ms_avg, 5),
+                     "median_launch_ms": round(statistics.median(decode_ms), 5)},
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(wl, pools[0], args.cpu_seconds)
+    print(json.dumps(result))
+
+
+def cpu_baseline(wl, pool, budget_s):
+    """The CPU oracle on a bounded sample: the first n sequences of the same
+    batch (same block tables, same pools), median of >= 3 repetitions."""
+    import torch
+    from oracle import paged as oracle_paged
+    kp, vp = pool[0].cpu(), pool[1].cpu()
+    q, bt, cl = wl.query.cpu(), wl.block_tables.cpu(), wl.context_lens.cpu()
+    n = min(wl.batch, 8)
+    t0 = time.perf_counter()
+    oracle_paged.paged_decode(q[:n], kp, vp, bt[:n], cl[:n])       # warm-up, also sizes the sample
+    per_seq = (time.perf_counter() - t0) / n
+    n = int(max(1, min(wl.batch, budget_s / 4 / max(per_seq, 1e-6))))
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle_paged.paged_decode(q[:n], kp, vp, bt[:n], cl[:n])
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    tokens = int(cl[:n].sum())
+    nbytes = tokens * wl.kv_bytes_per_token()
+    try:
+        model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
+    except Exception:
+        model = "unknown"
+    return {"value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"first {n} of {wl.batch} sequences of the same batch, one layer, "
+            f"median of 3 (after 1 warm-up); {tokens} context tokens",
+            "tokens_per_s_per_layer": round(n / t, 2), "host_cpu_count": os.cpu_count(), "cpu_model": model}
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,159 @@
+/*
+ * ironcore_paged.h -- C ABI of the MI355X (gfx950) paged-attention library.
+ *
+ * The reference (haanjack/ironcore) has no FFI, no KV cache and no native
+ * code: its attention boundary is the Python call
+ *     Attention.forward(query, key, value, attention_mask=None)
+ *         ironcore/layers/attention.py:208-253
+ * made from TransformerLayer.custom_forward
+ *         ironcore/models/transformer.py:101-103
+ * Each entry point below names the reference code whose work it takes over
+ * when that call runs against a block KV cache.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer borrowed for the duration of the call
+ *    (the kernels are enqueued on `stream`; the memory must stay valid until
+ *    the stream reaches them).  The library never allocates or frees.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *  - Return value: IC_OK (0) or a negative IC_ERR_* code.  Argument errors
+ *    are detected on the host before anything is launched.  The library
+ *    never throws, never exits the process and keeps no mutable global
+ *    state, so calls may come from any host thread; ordering is the
+ *    stream's.
+ *  - Element type is selected by `dtype` (IC_DTYPE_*).  Strides are in
+ *    ELEMENTS.  The head dimension is always contiguous.
+ *
+ * Block KV cache layout (defined by this library; the reference has none)
+ *  - k_pool, v_pool: num_blocks blocks of `block_size` tokens.  Element
+ *    (block, kv_head, token_in_block, d) lives at
+ *        block*pool_stride_block + kv_head*pool_stride_head
+ *        + token_in_block*pool_stride_token + d.
+ *    The native layout is [num_blocks, gn, block_size, hd] contiguous
+ *    (pool_stride_block = gn*block_size*hd, pool_stride_head = block_size*hd,
+ *    pool_stride_token = hd), which makes one (block, kv_head) tile a single
+ *    contiguous run of block_size*hd elements.
+ *  - block_tables: int32 [n_seqs, block_table_stride]; entry j of row i is
+ *    the pool block that holds tokens [j*block_size, (j+1)*block_size) of
+ *    sequence i.  Rows may alias blocks (shared prefixes).
+ *  - context_lens: int32 [n_seqs]; number of tokens visible to the query,
+ *    including tokens appended for this step.
+ *  - slot_mapping: int64 [n_tokens]; block*block_size + token_in_block for
+ *    each new K/V row; a negative slot marks a padding row and is skipped.
+ *  - GQA: query head h reads KV head h / (hn / gn)
+ *    (ironcore/layers/attention.py:95-102).
+ */
+#ifndef IRONCORE_PAGED_H
+#define IRONCORE_PAGED_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IC_OK                 0
+#define IC_ERR_NULL_POINTER  (-1)  /* a required pointer is NULL                 */
+#define IC_ERR_BAD_SHAPE     (-2)  /* a size/stride is non-positive or inconsistent */
+#define IC_ERR_UNSUPPORTED   (-3)  /* dtype / head_dim / group size / block size not built */
+#define IC_ERR_WORKSPACE     (-4)  /* workspace missing or too small             */
+#define IC_ERR_LAUNCH        (-5)  /* hipGetLastError() reported a launch failure */
+#define IC_ERR_ALIGNMENT     (-6)  /* a pointer or stride breaks the 16-byte rule */
+
+#define IC_DTYPE_BF16 0
+#define IC_DTYPE_F16  1
+#define IC_DTYPE_F32  2
+
+/* Library ABI version (major*10000 + minor*100 + patch). */
+int ic_version(void);
+
+/* Static, NUL-terminated description of an IC_* code. */
+const char *ic_error_string(int code);
+
+/*
+ * KV append: copy the K/V rows a transformer layer produced for n_tokens new
+ * tokens into their cache slots, bit for bit.  Replaces nothing in the
+ * reference (which recomputes K/V for the whole sequence every step,
+ * examples/generate_text.py:27); the rows are the `key`/`value` tensors of
+ * ironcore/models/transformer.py:88-98.
+ *
+ *   k_new, v_new   [n_tokens, gn, hd], row stride new_stride_token, heads and
+ *                  head_dim contiguous within a row
+ *   slot_mapping   int64 [n_tokens]
+ * Slots outside [0, num_blocks*block_size) are skipped.
+ */
+int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
+                 void *k_pool, void *v_pool,
+                 int64_t pool_stride_block, int64_t pool_stride_head,
+                 int64_t pool_stride_token,
+                 const int64_t *slot_mapping, int64_t n_tokens,
+                 int gn, int hd, int block_size, int64_t num_blocks,
+                 int dtype, void *stream);
+
+/*
+ * Workspace the decode entry point needs for its split-K partials, in bytes,
+ * for any call with these bounds (0 is never returned for valid arguments).
+ * part_tokens = 0 selects the library default.
+ */
+size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int hd,
+                                       int max_context_len, int part_tokens);
+
+/*
+ * Paged decode: one query token per sequence against the block KV cache.
+ * Computes what ironcore/layers/attention.py:68-142 (_attention) returns for
+ * sq = 1 on the rows the block table points at:
+ *     out[i, h*hd + d] = sum_j softmax_j(q[i,h] . k[i,j,h/G] * scale) * v[i,j,h/G,d]
+ *
+ *   out           [n_seqs, hn*hd], row stride out_stride_seq
+ *   q             [n_seqs, hn, hd], row stride q_stride_seq
+ *   scale         multiplies q.k (the reference divides by sqrt(hd),
+ *                 attention.py:65,110; pass 1/sqrt(hd))
+ *   max_context_len  upper bound on context_lens (sizes the split-K grid;
+ *                 larger entries are clamped to it)
+ *   part_tokens   tokens per split-K partition (multiple of block_size), 0 = default
+ *   workspace     at least ic_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
+ * Sequences with context_lens[i] <= 0 produce zeros.
+ */
+int ic_paged_decode(void *out, int64_t out_stride_seq,
+                    const void *q, int64_t q_stride_seq,
+                    const void *k_pool, const void *v_pool,
+                    int64_t pool_stride_block, int64_t pool_stride_head,
+                    int64_t pool_stride_token,
+                    const int32_t *block_tables, int64_t block_table_stride,
+                    const int32_t *context_lens,
+                    int n_seqs, int hn, int gn, int hd, int block_size,
+                    int64_t num_blocks, int max_context_len, float scale,
+                    int part_tokens, void *workspace, size_t workspace_bytes,
+                    int dtype, void *stream);
+
+/*
+ * Chunked prefill against the block KV cache: each sequence brings a chunk of
+ * new query tokens whose K/V rows are already appended; query row r of a
+ * chunk of length C in a sequence of context length L sees keys
+ * j <= (L - C) + r.  Computes what attention.py:68-142 returns for
+ * sq = C, sk = L with the causal mask of ironcore/language_model.py:109-114
+ * shifted by the cached prefix.  With causal = 0 every query row sees all L
+ * keys (the reference's attention_mask=None case).
+ *
+ *   out           [n_tokens, hn*hd], row stride out_stride_token
+ *   q             [n_tokens, hn, hd], row stride q_stride_token; the chunk of
+ *                 sequence i is rows cu_seqlens_q[i] .. cu_seqlens_q[i+1]-1
+ *   cu_seqlens_q  int32 [n_seqs + 1]
+ *   max_chunk_len upper bound on any chunk length (sizes the grid)
+ */
+int ic_paged_prefill(void *out, int64_t out_stride_token,
+                     const void *q, int64_t q_stride_token,
+                     const void *k_pool, const void *v_pool,
+                     int64_t pool_stride_block, int64_t pool_stride_head,
+                     int64_t pool_stride_token,
+                     const int32_t *block_tables, int64_t block_table_stride,
+                     const int32_t *context_lens, const int32_t *cu_seqlens_q,
+                     int n_seqs, int max_chunk_len,
+                     int hn, int gn, int hd, int block_size,
+                     int64_t num_blocks, float scale, int causal,
+                     int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IRONCORE_PAGED_H */

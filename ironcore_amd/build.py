@@ -1,0 +1,78 @@
+"""Build recipe for the HIP library: hipcc, gfx950 only, in-tree output.
+
+    python -m ironcore_amd.build
+
+compiles every translation unit under ironcore_amd/csrc/ and links
+ironcore_amd/lib/libironcore_paged.so.  Cross-compiles without a GPU.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+LIB_DIR = PKG / "lib"
+LIB_PATH = LIB_DIR / "libironcore_paged.so"
+OBJ_DIR = PKG / "build" / "obj"
+
+SOURCES = ["ic_api.hip", "kv_append.hip", "paged_decode.hip", "paged_prefill.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fno-gpu-rdc",
+    "-Wall",
+    "-Wno-unused-function",
+    # hipcc -O3 must not form packed-fp32 VALU ops on its own.
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the HIP library cannot be built")
+    return exe
+
+
+def _compile(src: str, extra: list[str]) -> Path:
+    obj = OBJ_DIR / (src + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")
+    noise = "is not a recognized feature for this target"
+    warn = "\n".join(line for line in res.stderr.splitlines() if noise not in line)
+    if warn.strip():
+        sys.stderr.write(warn + "\n")
+    return obj
+
+
+def build(verbose: bool = True, extra_flags: list[str] | None = None) -> Path:
+    """Compile and link; returns the path of the shared library."""
+    extra = list(extra_flags or [])
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(lambda s: _compile(s, extra), SOURCES))
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc",
+           *map(str, objs), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

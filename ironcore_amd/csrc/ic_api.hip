@@ -1,0 +1,189 @@
+// C ABI: argument validation on the host, then dispatch to the kernel
+// launchers.  Nothing here allocates, synchronises or keeps state.
+#include "ic_internal.h"
+#include "../../include/ironcore_paged.h"
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool dtype_ok(int dtype) { return dtype == IC_DTYPE_BF16 || dtype == IC_DTYPE_F16 || dtype == IC_DTYPE_F32; }
+
+// A stride (elements) keeps 16-byte chunks aligned when stride*elem % 16 == 0.
+bool stride16(int64_t stride, int es) { return ((stride * es) & 15) == 0; }
+
+int check_pool(int64_t sb, int64_t sh, int64_t st, int gn, int hd, int block_size, int64_t num_blocks,
+               int es) {
+  if (gn <= 0 || hd <= 0 || block_size <= 0 || num_blocks <= 0) return IC_ERR_BAD_SHAPE;
+  if (sb <= 0 || sh <= 0 || st < hd) return IC_ERR_BAD_SHAPE;
+  if ((hd * es) % 16 != 0) return IC_ERR_UNSUPPORTED;
+  if (!stride16(sb, es) || !stride16(sh, es) || !stride16(st, es)) return IC_ERR_ALIGNMENT;
+  return IC_OK;
+}
+
+int resolve_part_tokens(int part_tokens, int block_size) {
+  if (part_tokens == 0) part_tokens = ic::kDefaultPartTokens;
+  if (part_tokens < block_size || part_tokens % block_size != 0) return -1;
+  if (part_tokens / block_size > ic::kMaxPartBlocks) return -1;
+  return part_tokens;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ic_version(void) { return 100; }
+
+const char *ic_error_string(int code) {
+  switch (code) {
+    case IC_OK: return "ok";
+    case IC_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case IC_ERR_BAD_SHAPE: return "a size or stride is non-positive or inconsistent";
+    case IC_ERR_UNSUPPORTED: return "no kernel built for this dtype / head_dim / group / block size";
+    case IC_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case IC_ERR_LAUNCH: return "kernel launch failed";
+    case IC_ERR_ALIGNMENT: return "pointer or stride is not 16-byte aligned";
+    default: return "unknown error code";
+  }
+}
+
+int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token, void *k_pool,
+                 void *v_pool, int64_t pool_stride_block, int64_t pool_stride_head,
+                 int64_t pool_stride_token, const int64_t *slot_mapping, int64_t n_tokens, int gn,
+                 int hd, int block_size, int64_t num_blocks, int dtype, void *stream) {
+  if (n_tokens < 0) return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                          num_blocks, es))
+    return rc;
+  if (n_tokens == 0) return IC_OK;
+  if (!k_new || !v_new || !k_pool || !v_pool || !slot_mapping) return IC_ERR_NULL_POINTER;
+  if (new_stride_token < (int64_t)gn * hd) return IC_ERR_BAD_SHAPE;
+  if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_pool) || !aligned16(v_pool) ||
+      !stride16(new_stride_token, es))
+    return IC_ERR_ALIGNMENT;
+  ic::AppendArgs a;
+  a.k_new = k_new;
+  a.v_new = v_new;
+  a.new_stride_token = new_stride_token;
+  a.k_pool = k_pool;
+  a.v_pool = v_pool;
+  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
+  a.slot_mapping = slot_mapping;
+  a.n_tokens = n_tokens;
+  a.gn = gn;
+  a.hd = hd;
+  a.dtype = dtype;
+  return ic::launch_kv_append(a, static_cast<hipStream_t>(stream));
+}
+
+size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int hd, int max_context_len,
+                                       int part_tokens) {
+  if (n_seqs <= 0 || hn <= 0 || hd <= 0 || max_context_len <= 0) return 0;
+  if (part_tokens == 0) part_tokens = ic::kDefaultPartTokens;
+  if (part_tokens < 0) return 0;
+  const size_t n_parts = ((size_t)max_context_len + part_tokens - 1) / part_tokens;
+  const size_t slots = (size_t)n_seqs * hn * n_parts;
+  const size_t ml = (slots * 2 * sizeof(float) + 255) & ~(size_t)255;
+  return ml + slots * hd * sizeof(float);
+}
+
+int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
+                    const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                    int64_t pool_stride_head, int64_t pool_stride_token, const int32_t *block_tables,
+                    int64_t block_table_stride, const int32_t *context_lens, int n_seqs, int hn,
+                    int gn, int hd, int block_size, int64_t num_blocks, int max_context_len,
+                    float scale, int part_tokens, void *workspace, size_t workspace_bytes, int dtype,
+                    void *stream) {
+  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0) return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                          num_blocks, es))
+    return rc;
+  if (n_seqs == 0) return IC_OK;
+  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
+  if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
+  if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
+  const int pt = resolve_part_tokens(part_tokens, block_size);
+  if (pt < 0) return IC_ERR_BAD_SHAPE;
+  const int64_t need_blocks = ((int64_t)max_context_len + block_size - 1) / block_size;
+  if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !stride16(q_stride_seq, es))
+    return IC_ERR_ALIGNMENT;
+  const size_t need = ic_paged_decode_workspace_bytes(n_seqs, hn, hd, max_context_len, pt);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return IC_ERR_WORKSPACE;
+
+  ic::DecodeArgs a;
+  a.out = out;
+  a.out_stride_seq = out_stride_seq;
+  a.q = q;
+  a.q_stride_seq = q_stride_seq;
+  a.k_pool = k_pool;
+  a.v_pool = v_pool;
+  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
+  a.block_tables = block_tables;
+  a.block_table_stride = block_table_stride;
+  a.context_lens = context_lens;
+  a.n_seqs = n_seqs;
+  a.hn = hn;
+  a.gn = gn;
+  a.hd = hd;
+  a.max_context_len = max_context_len;
+  a.scale = scale;
+  a.part_tokens = pt;
+  a.n_parts = (max_context_len + pt - 1) / pt;
+  const size_t slots = (size_t)n_seqs * hn * a.n_parts;
+  a.part_ml = static_cast<float *>(workspace);
+  a.part_acc = reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                         ((slots * 2 * sizeof(float) + 255) & ~(size_t)255));
+  a.dtype = dtype;
+  return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
+}
+
+int ic_paged_prefill(void *out, int64_t out_stride_token, const void *q, int64_t q_stride_token,
+                     const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                     int64_t pool_stride_head, int64_t pool_stride_token,
+                     const int32_t *block_tables, int64_t block_table_stride,
+                     const int32_t *context_lens, const int32_t *cu_seqlens_q, int n_seqs,
+                     int max_chunk_len, int hn, int gn, int hd, int block_size, int64_t num_blocks,
+                     float scale, int causal, int dtype, void *stream) {
+  if (n_seqs < 0 || max_chunk_len < 0 || hn <= 0 || gn <= 0 || hn % gn != 0) return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                          num_blocks, es))
+    return rc;
+  if (n_seqs == 0 || max_chunk_len == 0) return IC_OK;
+  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens || !cu_seqlens_q)
+    return IC_ERR_NULL_POINTER;
+  if (out_stride_token < (int64_t)hn * hd || q_stride_token < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
+  if (block_table_stride <= 0) return IC_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(out) || !aligned16(k_pool) || !aligned16(v_pool) ||
+      !stride16(q_stride_token, es) || !stride16(out_stride_token, es))
+    return IC_ERR_ALIGNMENT;
+  ic::PrefillArgs a;
+  a.out = out;
+  a.out_stride_token = out_stride_token;
+  a.q = q;
+  a.q_stride_token = q_stride_token;
+  a.k_pool = k_pool;
+  a.v_pool = v_pool;
+  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
+  a.block_tables = block_tables;
+  a.block_table_stride = block_table_stride;
+  a.context_lens = context_lens;
+  a.cu_seqlens_q = cu_seqlens_q;
+  a.n_seqs = n_seqs;
+  a.max_chunk_len = max_chunk_len;
+  a.hn = hn;
+  a.gn = gn;
+  a.hd = hd;
+  a.scale = scale;
+  a.causal = causal;
+  a.dtype = dtype;
+  return ic::launch_paged_prefill(a, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,178 @@
+"""Tensor-level wrappers over the C ABI: shape checks, strides, stream.
+
+Every function here runs the hand-written HIP kernels on the tensors' GPU, on
+torch's current stream.  CPU tensors are rejected: the paged path has no
+non-HIP implementation.
+
+Pool layout: ``k_pool``/``v_pool`` are ``[num_blocks, gn, block_size, hd]``
+(any strides with a contiguous last dimension); token ``p`` of sequence ``i``
+is ``pool[block_tables[i, p // block_size], :, p % block_size, :]``.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("paged attention runs on the GPU only (got a tensor on "
+                               f"{t.device}); there is no CPU path")
+        if t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _pool_strides(k_pool: torch.Tensor, v_pool: torch.Tensor):
+    if k_pool.dim() != 4 or k_pool.shape != v_pool.shape or k_pool.stride() != v_pool.stride():
+        raise ValueError("k_pool and v_pool must be [num_blocks, gn, block_size, hd] with equal strides")
+    if k_pool.stride(3) != 1:
+        raise ValueError("the head dimension of the pools must be contiguous")
+    nb, gn, bs, hd = k_pool.shape
+    sb, sh, st, _ = k_pool.stride()
+    return nb, gn, bs, hd, sb, sh, st
+
+
+class _Workspace:
+    """Split-K scratch, grown on demand, one per device.  Kernels that use it
+    are stream-ordered, so reuse across calls on one stream is safe."""
+
+    def __init__(self):
+        self._buf: dict[torch.device, torch.Tensor] = {}
+
+    def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
+        buf = self._buf.get(device)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+            self._buf[device] = buf
+        return buf
+
+
+_workspace = _Workspace()
+
+
+def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+              slot_mapping: torch.Tensor) -> None:
+    """Copy rows ``k_new[t]``, ``v_new[t]`` (``[n, gn, hd]``) into pool slot
+    ``slot_mapping[t]`` (= block*block_size + offset), bit for bit.  Negative
+    slots are skipped."""
+    lib = _lib.load()
+    dev = _require_gpu(k_new, v_new, k_pool, v_pool, slot_mapping)
+    nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
+    if k_new.dim() != 3 or k_new.shape != v_new.shape or tuple(k_new.shape[1:]) != (gn, hd):
+        raise ValueError(f"k_new/v_new must be [n, {gn}, {hd}], got {tuple(k_new.shape)} / {tuple(v_new.shape)}")
+    if k_new.dtype != k_pool.dtype or v_new.dtype != k_pool.dtype:
+        raise TypeError("new rows and pools must share a dtype")
+    n = k_new.shape[0]
+    if slot_mapping.dtype != torch.int64 or slot_mapping.numel() != n or not slot_mapping.is_contiguous():
+        raise ValueError("slot_mapping must be a contiguous int64 tensor with one slot per new row")
+
+    def rows_ok(t):
+        return t.stride(2) == 1 and t.stride(1) == hd
+    if not (rows_ok(k_new) and rows_ok(v_new) and k_new.stride(0) == v_new.stride(0)):
+        k_new, v_new = k_new.contiguous(), v_new.contiguous()
+    with torch.cuda.device(dev):
+        rc = lib.ic_kv_append(k_new.data_ptr(), v_new.data_ptr(), k_new.stride(0),
+                              k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                              slot_mapping.data_ptr(), n, gn, hd, bs, nb,
+                              _lib.dtype_code(k_pool.dtype), _lib.current_stream_ptr(dev))
+    _lib.check("ic_kv_append", rc)
+
+
+def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                 block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
+                 scale: float | None = None, out: torch.Tensor | None = None,
+                 part_tokens: int = 0) -> torch.Tensor:
+    """One query token per sequence.  ``query`` ``[b, hn, hd]`` -> ``[b, hn*hd]``.
+
+    ``max_context_len`` is a host-side upper bound on ``context_lens`` (it
+    sizes the split-K grid without a device synchronisation)."""
+    lib = _lib.load()
+    dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens)
+    nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
+    if query.dim() != 3 or query.shape[2] != hd:
+        raise ValueError(f"query must be [b, hn, {hd}], got {tuple(query.shape)}")
+    if query.dtype != k_pool.dtype:
+        raise TypeError("query and pools must share a dtype")
+    b, hn, _ = query.shape
+    if hn % gn != 0:
+        raise ValueError(f"{hn} query heads are not a multiple of {gn} KV heads")
+    if query.stride(2) != 1 or query.stride(1) != hd:
+        query = query.contiguous()
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] != b \
+            or block_tables.stride(1) != 1:
+        raise ValueError("block_tables must be int32 [b, max_blocks] with contiguous rows")
+    if context_lens.dtype != torch.int32 or context_lens.numel() != b or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous int32 [b] tensor")
+    max_context_len = int(max_context_len)
+    if max_context_len > block_tables.shape[1] * bs:
+        raise ValueError("max_context_len exceeds what the block table can address")
+    if out is None:
+        out = torch.empty(b, hn * hd, dtype=query.dtype, device=dev)
+    elif out.shape != (b, hn * hd) or out.dtype != query.dtype or out.stride(1) != 1:
+        raise ValueError("out must be [b, hn*hd] in the query dtype with contiguous rows")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    need = lib.ic_paged_decode_workspace_bytes(b, hn, hd, max(max_context_len, 1), part_tokens)
+    ws = _workspace.get(dev, need)
+    with torch.cuda.device(dev):
+        rc = lib.ic_paged_decode(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                 k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                 block_tables.data_ptr(), block_tables.stride(0),
+                                 context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
+                                 float(scale), part_tokens, ws.data_ptr(), ws.numel(),
+                                 _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+    _lib.check("ic_paged_decode", rc)
+    return out
+
+
+def paged_prefill(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                  block_tables: torch.Tensor, context_lens: torch.Tensor,
+                  cu_seqlens_q: torch.Tensor, max_chunk_len: int, causal: bool = True,
+                  scale: float | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Chunked prefill.  ``query`` is the flat ``[n_tokens, hn, hd]``
+    concatenation of the sequences' new chunks (chunk ``i`` = rows
+    ``cu_seqlens_q[i]:cu_seqlens_q[i+1]``); the chunk's K/V are already in the
+    pool and ``context_lens[i]`` counts prefix + chunk.  -> ``[n_tokens, hn*hd]``."""
+    lib = _lib.load()
+    dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens, cu_seqlens_q)
+    nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
+    if query.dim() != 3 or query.shape[2] != hd:
+        raise ValueError(f"query must be [n_tokens, hn, {hd}], got {tuple(query.shape)}")
+    if query.dtype != k_pool.dtype:
+        raise TypeError("query and pools must share a dtype")
+    n_tokens, hn, _ = query.shape
+    if hn % gn != 0:
+        raise ValueError(f"{hn} query heads are not a multiple of {gn} KV heads")
+    if query.stride(2) != 1 or query.stride(1) != hd:
+        query = query.contiguous()
+    n_seqs = context_lens.numel()
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] != n_seqs \
+            or block_tables.stride(1) != 1:
+        raise ValueError("block_tables must be int32 [n_seqs, max_blocks] with contiguous rows")
+    if context_lens.dtype != torch.int32 or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous int32 tensor")
+    if cu_seqlens_q.dtype != torch.int32 or cu_seqlens_q.numel() != n_seqs + 1 \
+            or not cu_seqlens_q.is_contiguous():
+        raise ValueError("cu_seqlens_q must be a contiguous int32 [n_seqs + 1] tensor")
+    if out is None:
+        out = torch.empty(n_tokens, hn * hd, dtype=query.dtype, device=dev)
+    elif out.shape != (n_tokens, hn * hd) or out.dtype != query.dtype or out.stride(1) != 1:
+        raise ValueError("out must be [n_tokens, hn*hd] in the query dtype with contiguous rows")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    with torch.cuda.device(dev):
+        rc = lib.ic_paged_prefill(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                  k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                  block_tables.data_ptr(), block_tables.stride(0),
+                                  context_lens.data_ptr(), cu_seqlens_q.data_ptr(), n_seqs,
+                                  int(max_chunk_len), hn, gn, hd, bs, nb, float(scale),
+                                  1 if causal else 0, _lib.dtype_code(query.dtype),
+                                  _lib.current_stream_ptr(dev))
+    _lib.check("ic_paged_prefill", rc)
+    return out

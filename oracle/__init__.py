@@ -1,0 +1,41 @@
+"""CPU oracle for the paged-attention path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing under this package is part of the shipped product: only the test
+suite, the smoke check and the CPU-baseline leg of the benchmark may import
+it, and only as the checker.  The product package never imports it.
+
+Contents
+--------
+dense_attention   torch restatement of the reference's dense attention
+                  arithmetic (ironcore/layers/attention.py:68-142), same ops,
+                  same order, same dtype at every step.
+paged             block-table gather + KV-append closed form that drive the
+                  dense restatement through a block KV cache (the cache
+                  interface is defined by this build; the reference has none).
+brute_force       independent float64 loops used to pin dense_attention.
+gpt2              CPU restatement of the reference's GPT-2-shaped forward
+                  (ironcore/language_model.py:67-100, ironcore/models/
+                  transformer.py:77-132) with a full-recompute generate loop
+                  and a block-KV-cache generate loop.
+
+Pinning status (what checks each function; see tests/test_oracle_*.py)
+-----------------------------------------------------------------------
+dense_attention.dense_attention   pinned: float64 brute force on tiny shapes,
+                                  torch scaled_dot_product_attention in fp32,
+                                  closed forms (ctx=1, equal keys, shift
+                                  invariance), GQA == MHA on repeated K/V.
+                                  The reference's tests hold no golden vectors
+                                  for it (shape/finiteness checks only).
+paged.gather_kv / paged_decode /
+  paged_prefill                   pinned: block-permutation invariance, equals
+                                  dense over contiguous rows, chunked prefill
+                                  equals rows [P, P+C) of one causal pass.
+paged.kv_append                   pinned: closed form vs torch index_copy_,
+                                  sentinel preservation, idempotence.
+gpt2.*                            pinned: cached generate == full recompute
+                                  (causal-model identity); layer arithmetic vs
+                                  torch.nn.functional primitives.
+_flash_attention numerics         parity unpinned (third-party flash_attn wheel,
+                                  absent here; ironcore/layers/attention.py:
+                                  144-206).  Not restated.
+"""

@@ -1,0 +1,123 @@
+"""Paged decode through the C ABI against the CPU oracle (the reference's
+dense attention on the gathered rows).  Tolerance: max-abs 2e-2 in bf16/fp16
+(the bound the target states), 1e-4 in fp32."""
+import pytest
+import torch
+
+from ironcore_amd import paged_ops, workloads
+from oracle import paged as oracle_paged
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 2e-2, torch.float32: 1e-4}
+
+
+def _run(wl, gpu, **kw):
+    d = wl.to(gpu)
+    out = paged_ops.paged_decode(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens,
+                                 d.max_context_len, **kw)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _oracle(wl):
+    return oracle_paged.paged_decode(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens)
+
+
+def _check(wl, out, tol=None):
+    ref = _oracle(wl)
+    tol = tol or TOL[wl.query.dtype]
+    diff = (out.float() - ref.float()).abs().max().item()
+    assert torch.isfinite(out.float()).all()
+    assert diff <= tol, f"max|diff| {diff} > {tol} ({wl.name})"
+    return diff
+
+
+@pytest.mark.parametrize("hn,gn", [(32, 32), (64, 8), (28, 4), (8, 4), (12, 4), (5, 1), (6, 1), (24, 1)])
+def test_decode_group_sizes_bf16(gpu, hn, gn):
+    wl = workloads.make_decode_workload(6, hn, gn, 128, 1, 1300, seed=hn * 100 + gn)
+    _check(wl, _run(wl, gpu))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hd", [64, 128])
+def test_decode_dtypes_head_dims(gpu, dtype, hd):
+    wl = workloads.make_decode_workload(5, 8, 4, hd, 1, 900, dtype=dtype, seed=hd)
+    _check(wl, _run(wl, gpu))
+
+
+@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 511, 512, 513, 1024, 1025])
+def test_decode_boundary_lengths(gpu, ctx):
+    wl = workloads.make_decode_workload(3, 4, 2, 128, ctx, ctx, seed=ctx)
+    _check(wl, _run(wl, gpu))
+
+
+def test_decode_ctx1_returns_value_row(gpu):
+    """One cached token: softmax is 1, so the output is that token's V row, bit for bit."""
+    wl = workloads.make_decode_workload(4, 8, 2, 128, 1, 1, seed=11)
+    out = _run(wl, gpu)
+    for i in range(4):
+        v = wl.v_pool[wl.block_tables[i, 0].long(), :, 0, :]          # [gn, hd]
+        want = v.repeat_interleave(4, dim=0).reshape(-1)
+        assert torch.equal(out[i].view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("part_tokens", [16, 64, 256, 512, 1024, 4096])
+def test_decode_split_invariance(gpu, part_tokens):
+    wl = workloads.make_decode_workload(4, 8, 8, 128, 900, 2100, seed=5)
+    out = _run(wl, gpu, part_tokens=part_tokens)
+    _check(wl, out)
+    base = _run(wl, gpu, part_tokens=4096)      # one partition per sequence
+    assert (out.float() - base.float()).abs().max().item() <= 4e-3
+
+
+def test_decode_garbage_in_unused_slots(gpu):
+    """NaN/Inf bit patterns beyond the context length and in unused blocks must not leak."""
+    wl = workloads.make_decode_workload(4, 8, 4, 128, 5, 200, seed=9, extra_blocks=3)
+    ref = _oracle(wl)
+    nan = torch.tensor(float("nan"), dtype=torch.bfloat16)
+    for i in range(4):
+        ctx = int(wl.context_lens[i])
+        last = wl.block_tables[i, (ctx - 1) // 16].long()
+        used = (ctx - 1) % 16 + 1
+        wl.k_pool[last, :, used:, :] = nan
+        wl.v_pool[last, :, used:, :] = nan
+    out = _run(wl, gpu)
+    assert torch.isfinite(out.float()).all()
+    assert (out.float() - ref.float()).abs().max().item() <= 2e-2
+
+
+def test_decode_block_permutation_invariance(gpu):
+    wl = workloads.make_decode_workload(4, 8, 4, 128, 100, 700, seed=21)
+    out1 = _run(wl, gpu)
+    nb = wl.k_pool.shape[0]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(1))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(nb)
+    wl2 = workloads.DecodeWorkload(**{**wl.__dict__})
+    wl2.k_pool = wl.k_pool[perm]
+    wl2.v_pool = wl.v_pool[perm]
+    wl2.block_tables = inv[wl.block_tables.long()].to(torch.int32)
+    out2 = _run(wl2, gpu)
+    assert torch.equal(out1.view(torch.int16), out2.view(torch.int16))
+
+
+def test_decode_grpo_shared_prefix(gpu):
+    wl = workloads.make_grpo_workload(3, 4, 28, 4, 128, 128, 1, 200, seed=2)
+    _check(wl, _run(wl, gpu))
+
+
+def test_decode_empty_sequence_and_batch(gpu):
+    wl = workloads.make_decode_workload(3, 4, 4, 128, 10, 40, seed=4)
+    wl.context_lens[1] = 0
+    out = _run(wl, gpu)
+    assert torch.count_nonzero(out[1]) == 0
+    ref = _oracle(workloads.DecodeWorkload(**{**wl.__dict__, "context_lens": wl.context_lens.clamp(min=1)}))
+    assert (out[0].float() - ref[0].float()).abs().max().item() <= 2e-2
+    assert (out[2].float() - ref[2].float()).abs().max().item() <= 2e-2
+
+
+def test_decode_scaled_llama7b_slice(gpu):
+    """The headline shape at reduced batch: Llama-7B heads, contexts in [512, 4096]."""
+    wl = workloads.make_decode_workload(4, 32, 32, 128, 512, 4096, seed=0)
+    _check(wl, _run(wl, gpu))
