@@ -133,7 +133,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl.name, "batch": b, "q_heads": hn, "kv_heads": gn, "head_dim": hd,
                    "block_size": bs, "sum_context": wl.logical_tokens, "unique_tokens": wl.unique_tokens,
-                   "resident_layers": len(pools), "part_tokens": args.part_tokens or 512,
+                   "resident_layers": len(pools), "part_tokens": args.part_tokens or 256,
                    "step": "kv_append(64 rows) + paged_decode, one layer"},
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,

@@ -82,8 +82,8 @@ int launch_kv_append(const AppendArgs &a, hipStream_t stream);
 int launch_paged_decode(const DecodeArgs &a, hipStream_t stream);
 int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream);
 
-constexpr int kDefaultPartTokens = 512;
-constexpr int kMaxPartBlocks = 256;  // block-table entries staged in LDS per workgroup
+constexpr int kDefaultPartTokens = 256;
+constexpr int kMaxPartBlocks = 64;  // blocks per split-K partition: one block-table entry per lane
 
 inline int elem_size(int dtype) { return dtype == 2 ? 4 : 2; }
 

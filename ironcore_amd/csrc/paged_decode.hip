@@ -64,18 +64,32 @@ struct DecodeKP {
 
 constexpr float kNegInf = -__builtin_huge_valf();
 
+// One WAVE owns one split-K partition of one (sequence, KV head): the waves
+// of a workgroup never synchronise with each other, so a wave that finishes
+// (or has no tokens) retires on its own and the CU always has other waves'
+// loads in flight.  NW only sets how many partitions share a workgroup slot.
+#ifndef IC_DECODE_NW
+#define IC_DECODE_NW 4
+#endif
+#ifdef IC_DECODE_WAVES_PER_EU
+#define IC_DECODE_OCC __attribute__((amdgpu_waves_per_eu(IC_DECODE_WAVES_PER_EU)))
+#else
+#define IC_DECODE_OCC
+#endif
+
 template <class E, int HD, int GT, int BS, int NW>
-__global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP p) {
+__global__ __launch_bounds__(NW *kWave) IC_DECODE_OCC void paged_decode_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int EPL = E::EPL;
   constexpr int ES = sizeof(T);
   constexpr int LPR = HD / EPL;     // lanes sharing one token row
   constexpr int RPL = kWave / LPR;  // token rows per load instruction
   constexpr int NLD = BS / RPL;     // load instructions per (block, head) tile
-  constexpr int NGRP = NW * RPL;    // lane groups per workgroup
   static_assert(HD % EPL == 0 && kWave % LPR == 0 && BS % RPL == 0, "tile shape");
 
-  const int part = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int part = blockIdx.x * NW + wave;
   const int kvh = blockIdx.y / p.nsub;
   const int sub = blockIdx.y - kvh * p.nsub;
   const int seq = blockIdx.z;
@@ -86,43 +100,32 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   if (tok_begin >= ctx) return;
   const int tok_end = (tok_begin + p.part_tokens < ctx) ? tok_begin + p.part_tokens : ctx;
   const int blk_begin = tok_begin / BS;
-  const int nblk = (tok_end - tok_begin + BS - 1) / BS;
+  const int nblk = (tok_end - tok_begin + BS - 1) / BS;  // <= 64 (checked on the host)
   const int n_parts_seq = (ctx + p.part_tokens - 1) / p.part_tokens;
 
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;
   const int col = lane % LPR;
   const int rowg = lane / LPR;
-  const int head0 = kvh * p.group + sub * GT;  // first query head of this workgroup
+  const int head0 = kvh * p.group + sub * GT;  // first query head of this wave
   const int heads_here = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
 
-  __shared__ int32_t s_tbl[kMaxPartBlocks];
-  __shared__ __attribute__((aligned(16))) T s_q[GT * HD];
-  __shared__ float s_m[NGRP][GT];
-  __shared__ float s_l[NGRP][GT];
-  __shared__ float s_w[NGRP][GT];
-  __shared__ __attribute__((aligned(16))) float s_acc[NGRP][GT][HD];
-
-  for (int i = tid; i < nblk; i += NW * kWave) {
-    int32_t b = p.block_tables[seq * p.bt_stride + blk_begin + i];
+  // Lane i keeps the pool block of the partition's i-th block; the loop reads
+  // it back as a wave-uniform scalar (v_readlane), so tile addresses are SALU
+  // work and the table never sits on the load path again.
+  int32_t my_block = 0;
+  if (lane < nblk) {
+    my_block = p.block_tables[seq * p.bt_stride + blk_begin + lane];
     // A corrupt table entry must not become an out-of-pool address.
-    b = b < 0 ? 0 : b;
-    b = (int64_t)b >= p.num_blocks ? (int32_t)(p.num_blocks - 1) : b;
-    s_tbl[i] = b;
+    my_block = my_block < 0 ? 0 : my_block;
+    my_block = (int64_t)my_block >= p.num_blocks ? (int32_t)(p.num_blocks - 1) : my_block;
   }
-  for (int c = tid; c < GT * LPR; c += NW * kWave) {
-    const int g = c / LPR;
-    Vec16 v = {{0u, 0u, 0u, 0u}};
-    if (g < heads_here)
-      v = load16(p.q + (seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + (c - g * LPR) * EPL) * ES);
-    store16(&s_q[c * EPL], v);
-  }
-  __syncthreads();
 
   Vec16 qreg[GT];
 #pragma unroll
-  for (int g = 0; g < GT; ++g) qreg[g] = load16(&s_q[g * HD + col * EPL]);
+  for (int g = 0; g < GT; ++g) {
+    qreg[g] = Vec16{{0u, 0u, 0u, 0u}};
+    if (g < heads_here)
+      qreg[g] = load16(p.q + (seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + col * EPL) * ES);
+  }
 
   uint32_t lane_off[NLD];
 #pragma unroll
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   }
 
   auto issue = [&](int j, Vec16 *kk, Vec16 *vv) {
-    const int64_t phys = __builtin_amdgcn_readfirstlane(s_tbl[j]);
+    const int64_t phys = __builtin_amdgcn_readlane(my_block, j);
     const int64_t tile = (phys * p.stride_block + kvh * p.stride_head) * ES;
     const char *kb = p.k_pool + tile;
     const char *vb = p.v_pool + tile;
@@ -147,9 +150,15 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
     for (int i = 0; i < NLD; ++i) kk[i] = load16(kb + lane_off[i]);
 #pragma unroll
     for (int i = 0; i < NLD; ++i) vv[i] = load16(vb + lane_off[i]);
+    // Keep the loads ahead of the arithmetic that follows in program order:
+    // the scheduler would otherwise sink them below the current tile's work
+    // and shorten the prefetch distance.
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  auto consume = [&](int j, Vec16 *kk, Vec16 *vv) {
+  // `last` marks the partition's final tile, the only one that can be partly
+  // filled; every other tile skips the validity test.
+  auto consume = [&](int j, Vec16 *kk, Vec16 *vv, bool last) {
     const int tok0 = tok_begin + j * BS;
     float s[GT][NLD];
 #pragma unroll
@@ -160,7 +169,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
         s[g][i] = group_sum<LPR>(d) * p.scale_log2e;
       }
     }
-    if (tok0 + BS > tok_end) {  // last, partly filled block: hide the unused slots
+    if (last && tok0 + BS > tok_end) {  // partly filled block: hide the unused slots
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         if (tok0 + i * RPL + rowg >= tok_end) {
@@ -200,68 +209,71 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   };
 
   {
+    // Two register tiles in ping-pong.  The steady-state loop issues the next
+    // tile's loads unconditionally, so the wait before a tile is consumed
+    // covers that tile only and the prefetch stays in flight behind it.
     Vec16 ka[NLD], va[NLD], kb[NLD], vb[NLD];
-    int j = wave;
-    if (j < nblk) {
-      issue(j, ka, va);
-      while (true) {
-        if (j + NW < nblk) issue(j + NW, kb, vb);
-        consume(j, ka, va);
-        j += NW;
-        if (j >= nblk) break;
-        if (j + NW < nblk) issue(j + NW, ka, va);
-        consume(j, kb, vb);
-        j += NW;
-        if (j >= nblk) break;
-      }
+    int j = 0;
+    issue(0, ka, va);
+    for (; j + 2 < nblk; j += 2) {
+      issue(j + 1, kb, vb);
+      consume(j, ka, va, false);
+      issue(j + 2, ka, va);
+      consume(j + 1, kb, vb, false);
+    }
+    if (j + 2 == nblk) {
+      issue(j + 1, kb, vb);
+      consume(j, ka, va, false);
+      consume(j + 1, kb, vb, true);
+    } else {
+      consume(j, ka, va, true);
     }
   }
 
-  // ---- merge lane groups and waves (log-sum-exp combine) --------------------
-  const int grp = wave * RPL + rowg;
+  // ---- merge the RPL row groups of this wave (log-sum-exp combine) -----------
+  __shared__ __attribute__((aligned(16))) float s_acc[NW][RPL][GT][HD];
+  float lsum[GT], mall[GT];
 #pragma unroll
   for (int g = 0; g < GT; ++g) {
-    if (col == 0) {
-      s_m[grp][g] = m[g];
-      s_l[grp][g] = l[g];
-    }
+    float mx = m[g];
+    if (RPL >= 2) mx = fmaxf(mx, __shfl_xor(mx, LPR, kWave));
+    if (RPL >= 4) mx = fmaxf(mx, __shfl_xor(mx, 2 * LPR, kWave));
+    if (RPL >= 8) mx = fmaxf(mx, __shfl_xor(mx, 4 * LPR, kWave));
+    const float w = (m[g] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx);
+    float ls = l[g] * w;
+    if (RPL >= 2) ls += __shfl_xor(ls, LPR, kWave);
+    if (RPL >= 4) ls += __shfl_xor(ls, 2 * LPR, kWave);
+    if (RPL >= 8) ls += __shfl_xor(ls, 4 * LPR, kWave);
+    lsum[g] = ls;
+    mall[g] = mx;
 #pragma unroll
     for (int e = 0; e < EPL; e += 4) {
-      float4 v4 = make_float4(acc[g][e], acc[g][e + 1], acc[g][e + 2], acc[g][e + 3]);
-      *reinterpret_cast<float4 *>(&s_acc[grp][g][col * EPL + e]) = v4;
+      float4 v4 = make_float4(acc[g][e] * w, acc[g][e + 1] * w, acc[g][e + 2] * w, acc[g][e + 3] * w);
+      *reinterpret_cast<float4 *>(&s_acc[wave][rowg][g][col * EPL + e]) = v4;
     }
   }
-  __syncthreads();
-  for (int c = tid; c < NGRP * GT; c += NW * kWave) {
-    const int g = c % GT;
-    float mx = kNegInf;
-    for (int r = 0; r < NGRP; ++r) mx = fmaxf(mx, s_m[r][g]);
-    const float mine = s_m[c / GT][g];
-    s_w[c / GT][g] = (mine == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(mine - mx);
-  }
-  __syncthreads();
-  for (int o = tid; o < GT * HD; o += NW * kWave) {
-    const int g = o / HD;
-    const int d = o - g * HD;
-    if (g >= heads_here) continue;
-    float mx = kNegInf, lsum = 0.f, a = 0.f;
+  // Only this wave reads what it wrote: a wave-level LDS fence is enough.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int r = 0; r < NGRP; ++r) {
-      const float w = s_w[r][g];
-      mx = fmaxf(mx, s_m[r][g]);
-      lsum = __builtin_fmaf(s_l[r][g], w, lsum);
-      a = __builtin_fmaf(s_acc[r][g][d], w, a);
-    }
+  for (int g = 0; g < GT; ++g) {
+    if (g >= heads_here) break;
     const int h = head0 + g;
-    if (n_parts_seq == 1) {
-      reinterpret_cast<T *>(p.out)[seq * p.out_stride_seq + (int64_t)h * HD + d] = E::narrow(a / lsum);
-    } else {
-      const int64_t slot = ((int64_t)seq * p.hn + h) * p.n_parts + part;
-      p.part_acc[slot * HD + d] = a;
-      if (d == 0) {
-        p.part_ml[slot * 2] = mx;
-        p.part_ml[slot * 2 + 1] = lsum;
-      }
+    const int64_t slot = ((int64_t)seq * p.hn + h) * p.n_parts + part;
+#pragma unroll
+    for (int d = lane; d < HD; d += kWave) {
+      float a = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) a += s_acc[wave][r][g][d];
+      if (n_parts_seq == 1)
+        reinterpret_cast<T *>(p.out)[seq * p.out_stride_seq + (int64_t)h * HD + d] = E::narrow(a / lsum[g]);
+      else
+        p.part_acc[slot * HD + d] = a;
+    }
+    if (n_parts_seq != 1 && lane == 0) {
+      p.part_ml[slot * 2] = mall[g];
+      p.part_ml[slot * 2 + 1] = lsum[g];
     }
   }
 }
@@ -299,8 +311,8 @@ __global__ __launch_bounds__(HD) void paged_decode_reduce_kernel(const DecodeKP 
 template <class E, int HD, int GT>
 int launch_typed(const DecodeKP &kp, int gn, int n_seqs, hipStream_t stream) {
   constexpr int BS = 16;
-  constexpr int NW = 4;
-  dim3 grid(kp.n_parts, gn * kp.nsub, n_seqs);
+  constexpr int NW = IC_DECODE_NW;
+  dim3 grid((kp.n_parts + NW - 1) / NW, gn * kp.nsub, n_seqs);
   hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), grid, dim3(NW * kWave), 0, stream, kp);
   hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD>), dim3(kp.hn, n_seqs), dim3(HD), 0, stream, kp);
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;

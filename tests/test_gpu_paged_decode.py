@@ -62,12 +62,12 @@ def test_decode_ctx1_returns_value_row(gpu):
         assert torch.equal(out[i].view(torch.int16), want.view(torch.int16))
 
 
-@pytest.mark.parametrize("part_tokens", [16, 64, 256, 512, 1024, 4096])
+@pytest.mark.parametrize("part_tokens", [16, 64, 256, 512, 1024])
 def test_decode_split_invariance(gpu, part_tokens):
     wl = workloads.make_decode_workload(4, 8, 8, 128, 900, 2100, seed=5)
     out = _run(wl, gpu, part_tokens=part_tokens)
     _check(wl, out)
-    base = _run(wl, gpu, part_tokens=4096)      # one partition per sequence
+    base = _run(wl, gpu, part_tokens=1024)
     assert (out.float() - base.float()).abs().max().item() <= 4e-3
 
 
