@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=4, help="resident layer pools the steps rotate over")
-    ap.add_argument("--part-tokens", type=int, default=0, help="split-K partition size (0 = library default)")
+    ap.add_argument("--min-chunk-tokens", type=int, default=0, help="smallest split-K share (0 = library default)")
     ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
@@ -80,7 +80,7 @@ def main():
         kp, vp = pools[i % len(pools)]
         paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
         paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
-                               wl.max_context_len, out=out, part_tokens=args.part_tokens)
+                               wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens)
 
     # ---- parity gate on the tensors that are about to be timed --------------
     from oracle import paged as oracle_paged
@@ -105,7 +105,7 @@ def main():
         paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
         ev[i][0].record()
         paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
-                               wl.max_context_len, out=out, part_tokens=args.part_tokens)
+                               wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens)
         ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -133,7 +133,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl.name, "batch": b, "q_heads": hn, "kv_heads": gn, "head_dim": hd,
                    "block_size": bs, "sum_context": wl.logical_tokens, "unique_tokens": wl.unique_tokens,
-                   "resident_layers": len(pools), "part_tokens": args.part_tokens or 256,
+                   "resident_layers": len(pools),
                    "step": "kv_append(64 rows) + paged_decode, one layer"},
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,

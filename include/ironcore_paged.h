@@ -91,12 +91,11 @@ int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
                  int dtype, void *stream);
 
 /*
- * Workspace the decode entry point needs for its split-K partials, in bytes,
- * for any call with these bounds (0 is never returned for valid arguments).
- * part_tokens = 0 selects the library default.
+ * Workspace the decode entry point needs (block-count prefix sums and
+ * split-K partials), in bytes, for a batch of n_seqs sequences with these
+ * head counts.  Returns 0 for invalid arguments.
  */
-size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int hd,
-                                       int max_context_len, int part_tokens);
+size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd);
 
 /*
  * Paged decode: one query token per sequence against the block KV cache.
@@ -108,10 +107,13 @@ size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int hd,
  *   q             [n_seqs, hn, hd], row stride q_stride_seq
  *   scale         multiplies q.k (the reference divides by sqrt(hd),
  *                 attention.py:65,110; pass 1/sqrt(hd))
- *   max_context_len  upper bound on context_lens (sizes the split-K grid;
- *                 larger entries are clamped to it)
- *   part_tokens   tokens per split-K partition (multiple of block_size), 0 = default
- *   workspace     at least ic_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
+ *   max_context_len  upper bound on context_lens; larger entries are clamped
+ *                 to it, and block_table_stride must cover it
+ *   min_chunk_tokens  the K/V stream of the whole batch is cut into equal
+ *                 shares, one per resident wave (split-K); this is the
+ *                 smallest share (multiple of block_size), 0 = default
+ *   workspace     at least ic_paged_decode_workspace_bytes(...) bytes, 256-byte
+ *                 aligned; contents need not be initialised
  * Sequences with context_lens[i] <= 0 produce zeros.
  */
 int ic_paged_decode(void *out, int64_t out_stride_seq,
@@ -123,7 +125,7 @@ int ic_paged_decode(void *out, int64_t out_stride_seq,
                     const int32_t *context_lens,
                     int n_seqs, int hn, int gn, int hd, int block_size,
                     int64_t num_blocks, int max_context_len, float scale,
-                    int part_tokens, void *workspace, size_t workspace_bytes,
+                    int min_chunk_tokens, void *workspace, size_t workspace_bytes,
                     int dtype, void *stream);
 
 /*

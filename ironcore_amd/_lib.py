@@ -28,7 +28,7 @@ SIGNATURES = {
         c_void_p, c_int64,                      # slot_mapping, n_tokens
         c_int, c_int, c_int, c_int64,           # gn, hd, block_size, num_blocks
         c_int, c_void_p]),                      # dtype, stream
-    "ic_paged_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "ic_paged_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "ic_paged_decode": (c_int, [
         c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
         c_void_p, c_void_p,                     # k_pool, v_pool
@@ -36,7 +36,7 @@ SIGNATURES = {
         c_void_p, c_int64, c_void_p,            # block_tables, stride, context_lens
         c_int, c_int, c_int, c_int, c_int,      # n_seqs, hn, gn, hd, block_size
         c_int64, c_int, c_float,                # num_blocks, max_context_len, scale
-        c_int, c_void_p, c_size_t,              # part_tokens, workspace, workspace_bytes
+        c_int, c_void_p, c_size_t,              # min_chunk_tokens, workspace, workspace_bytes
         c_int, c_void_p]),                      # dtype, stream
     "ic_paged_prefill": (c_int, [
         c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride

@@ -1,5 +1,7 @@
 // C ABI: argument validation on the host, then dispatch to the kernel
 // launchers.  Nothing here allocates, synchronises or keeps state.
+#include <atomic>
+
 #include "ic_internal.h"
 #include "../../include/ironcore_paged.h"
 
@@ -20,14 +22,30 @@ int check_pool(int64_t sb, int64_t sh, int64_t st, int gn, int hd, int block_siz
   return IC_OK;
 }
 
-int resolve_part_tokens(int part_tokens, int block_size) {
-  if (part_tokens == 0) part_tokens = ic::kDefaultPartTokens;
-  if (part_tokens < block_size || part_tokens % block_size != 0) return -1;
-  if (part_tokens / block_size > ic::kMaxPartBlocks) return -1;
-  return part_tokens;
+int resolve_min_chunk(int min_chunk_tokens, int block_size) {
+  if (min_chunk_tokens == 0) min_chunk_tokens = ic::kDefaultMinChunkTokens;
+  if (min_chunk_tokens < block_size || min_chunk_tokens % block_size != 0) return -1;
+  return min_chunk_tokens;
 }
 
 }  // namespace
+
+namespace ic {
+
+int device_cu_count() {
+  static std::atomic<int> cache[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  int n = cache[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+      n = 256;
+    cache[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+}  // namespace ic
 
 extern "C" {
 
@@ -77,15 +95,9 @@ int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
   return ic::launch_kv_append(a, static_cast<hipStream_t>(stream));
 }
 
-size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int hd, int max_context_len,
-                                       int part_tokens) {
-  if (n_seqs <= 0 || hn <= 0 || hd <= 0 || max_context_len <= 0) return 0;
-  if (part_tokens == 0) part_tokens = ic::kDefaultPartTokens;
-  if (part_tokens < 0) return 0;
-  const size_t n_parts = ((size_t)max_context_len + part_tokens - 1) / part_tokens;
-  const size_t slots = (size_t)n_seqs * hn * n_parts;
-  const size_t ml = (slots * 2 * sizeof(float) + 255) & ~(size_t)255;
-  return ml + slots * hd * sizeof(float);
+size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd) {
+  if (n_seqs <= 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0) return 0;
+  return ic::decode_workspace(n_seqs, hn, gn, hd).total();
 }
 
 int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
@@ -93,8 +105,8 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
                     int64_t pool_stride_head, int64_t pool_stride_token, const int32_t *block_tables,
                     int64_t block_table_stride, const int32_t *context_lens, int n_seqs, int hn,
                     int gn, int hd, int block_size, int64_t num_blocks, int max_context_len,
-                    float scale, int part_tokens, void *workspace, size_t workspace_bytes, int dtype,
-                    void *stream) {
+                    float scale, int min_chunk_tokens, void *workspace, size_t workspace_bytes,
+                    int dtype, void *stream) {
   if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0) return IC_ERR_BAD_SHAPE;
   if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
   const int es = ic::elem_size(dtype);
@@ -105,14 +117,14 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
   if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
   if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
   if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
-  const int pt = resolve_part_tokens(part_tokens, block_size);
-  if (pt < 0) return IC_ERR_BAD_SHAPE;
+  const int mc = resolve_min_chunk(min_chunk_tokens, block_size);
+  if (mc < 0) return IC_ERR_BAD_SHAPE;
   const int64_t need_blocks = ((int64_t)max_context_len + block_size - 1) / block_size;
   if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;
   if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !stride16(q_stride_seq, es))
     return IC_ERR_ALIGNMENT;
-  const size_t need = ic_paged_decode_workspace_bytes(n_seqs, hn, hd, max_context_len, pt);
-  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+  const ic::DecodeWorkspace ws = ic::decode_workspace(n_seqs, hn, gn, hd);
+  if (!workspace || workspace_bytes < ws.total() || (reinterpret_cast<uintptr_t>(workspace) & 255u))
     return IC_ERR_WORKSPACE;
 
   ic::DecodeArgs a;
@@ -132,12 +144,11 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
   a.hd = hd;
   a.max_context_len = max_context_len;
   a.scale = scale;
-  a.part_tokens = pt;
-  a.n_parts = (max_context_len + pt - 1) / pt;
-  const size_t slots = (size_t)n_seqs * hn * a.n_parts;
-  a.part_ml = static_cast<float *>(workspace);
-  a.part_acc = reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                         ((slots * 2 * sizeof(float) + 255) & ~(size_t)255));
+  a.min_chunk_tokens = mc;
+  char *wsp = static_cast<char *>(workspace);
+  a.cum_blocks = reinterpret_cast<int32_t *>(wsp);
+  a.part_ml = reinterpret_cast<float *>(wsp + ws.cum_bytes);
+  a.part_acc = reinterpret_cast<float *>(wsp + ws.cum_bytes + ws.ml_bytes);
   a.dtype = dtype;
   return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
 }

@@ -47,10 +47,10 @@ struct DecodeArgs {
   int hd;
   int max_context_len;
   float scale;
-  int part_tokens;
-  int n_parts;     // ceil(max_context_len / part_tokens)
-  float *part_ml;  // [n_seqs, hn, n_parts, 2]
-  float *part_acc; // [n_seqs, hn, n_parts, hd]
+  int min_chunk_tokens;  // smallest split-K share (multiple of block_size)
+  int32_t *cum_blocks;   // workspace: [n_seqs + 1]
+  float *part_ml;        // workspace: [partial slots, 2]
+  float *part_acc;       // workspace: [partial slots, hd]
   int dtype;
 };
 
@@ -82,9 +82,36 @@ int launch_kv_append(const AppendArgs &a, hipStream_t stream);
 int launch_paged_decode(const DecodeArgs &a, hipStream_t stream);
 int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream);
 
-constexpr int kDefaultPartTokens = 256;
-constexpr int kMaxPartBlocks = 64;  // blocks per split-K partition: one block-table entry per lane
+constexpr int kDefaultMinChunkTokens = 128;
+// Upper bound on the waves of one decode launch (sizes the workspace): 8 waves
+// on each of the 4 SIMDs of up to 512 CUs.
+constexpr int kMaxDecodeWaves = 16384;
 
 inline int elem_size(int dtype) { return dtype == 2 ? 4 : 2; }
+
+// Query heads one wave carries for a KV head with `group` query heads; larger
+// groups are cut into ceil(group / 8) sub-groups.
+inline int decode_heads_per_wave(int group) { return group <= 8 ? group : 8; }
+
+// Split-K workspace layout for the decode entry point.
+struct DecodeWorkspace {
+  size_t cum_bytes;  // int32 [n_seqs + 1], padded to 256
+  size_t ml_bytes;   // float [slots, 2], padded to 256
+  size_t acc_bytes;  // float [slots, hd]
+  size_t total() const { return cum_bytes + ml_bytes + acc_bytes; }
+};
+inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd) {
+  const int group = hn / gn;
+  const int gt = decode_heads_per_wave(group);
+  const int nsub = (group + gt - 1) / gt;
+  // one partial per (wave, pair) segment: fewer than waves + pairs of them
+  const size_t slots = ((size_t)kMaxDecodeWaves + (size_t)n_seqs * gn * nsub) * gt;
+  auto pad = [](size_t n) { return (n + 255) & ~(size_t)255; };
+  return {pad(((size_t)n_seqs + 1) * sizeof(int32_t)), pad(slots * 2 * sizeof(float)),
+          slots * hd * sizeof(float)};
+}
+
+// Compute units of the current device (cached per device ordinal).
+int device_cu_count();
 
 }  // namespace ic

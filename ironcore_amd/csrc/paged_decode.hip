@@ -8,27 +8,35 @@
 //
 // HBM-bound streaming kernel (one pass over every visible K and V byte).
 //
-//  * grid = (split-K partition, kv head [x query sub-group], sequence).  A
-//    workgroup owns `part_tokens` consecutive tokens of one (sequence, KV
-//    head) and ALL G query heads that share that KV head, so each K/V byte
-//    is fetched once per KV head, not once per query head.
-//  * The partition's slice of the block table and the query group are staged
-//    in LDS once; block ids are then wave-uniform scalars.
-//  * A wave walks whole blocks.  One (block, kv head) tile is
-//    block_size*hd elements; each lane fetches 16 bytes per load, so one load
-//    instruction covers 1 KiB of consecutive tile bytes (64/LPR token rows,
-//    LPR = lanes per row).  The next tile's loads are issued before the
-//    current tile is consumed.
+//  * Unit of work: a TILE = one pool block (16 tokens) of one (sequence, KV
+//    head) "pair", for ALL G query heads that share the KV head, so each K/V
+//    byte is fetched once per KV head, not once per query head.  (G > 8 is
+//    cut into sub-groups of <= 8 heads, each its own pair.)
+//  * Split-K by equal shares: the tiles of the whole batch form one sequence
+//    (pair-major, block-minor); a plan kernel prefix-sums the per-sequence
+//    block counts, and every resident WAVE takes one contiguous chunk of
+//    ceil(N / waves) tiles.  A chunk may start and end inside a pair and may
+//    span several pairs; each (wave, pair) segment yields one partial.  All
+//    waves carry the same load whatever the spread of context lengths, the
+//    grid is exactly the number of waves the GPU holds at once, and waves
+//    never synchronise with each other.
+//  * Block ids of up to 64 blocks sit one per lane and are read back as
+//    wave-uniform scalars (v_readlane), so tile addresses are SALU work.
+//  * One tile is block_size*hd contiguous elements per K and per V; each lane
+//    fetches 16 bytes per load, so one load instruction covers 1 KiB of
+//    consecutive bytes (64/LPR token rows, LPR = lanes per row).  Two
+//    register tiles in ping-pong: the next tile's loads are in flight while
+//    the current one is consumed.
 //  * q.k: v_dot2 on the packed pairs, then a DPP butterfly over the LPR lanes
 //    that share a row.  Online softmax per lane group; p*v accumulates into
 //    EPL fp32 registers per query head with no cross-lane traffic.
-//  * Lane groups and waves are merged through LDS with a log-sum-exp
-//    combine.  A sequence that fits one partition is finished here;
-//    otherwise (m, l, acc) partials go to the workspace and the reduce kernel
-//    below combines them.
+//  * Segment end: the lane groups of the wave are merged (log-sum-exp) through
+//    a private LDS slab.  A segment that covers its whole pair writes the
+//    output row; otherwise (m, l, acc) go to the workspace and the reduce
+//    kernel combines the few partials of that pair.
 //
 // Algorithmic bytes per launch: sum_i ctx_i * 2 * gn * hd * elem (K and V,
-// once per KV head) + q, out, block-table slice and context lengths.
+// once per KV head) + q, out, block-table entries and context lengths.
 #include "ic_device.h"
 #include "ic_internal.h"
 #include "../../include/ironcore_paged.h"
@@ -44,8 +52,9 @@ struct DecodeKP {
   const int32_t *block_tables;
   const int32_t *context_lens;
   char *out;
-  float *part_ml;
-  float *part_acc;
+  int32_t *cum_blocks;  // [n_seqs + 1] exclusive prefix sum of per-sequence block counts
+  float *part_ml;       // [n_partials, GT, 2]
+  float *part_acc;      // [n_partials, GT, hd]
   int64_t q_stride_seq;    // elements
   int64_t out_stride_seq;  // elements
   int64_t stride_block;    // elements
@@ -53,78 +62,100 @@ struct DecodeKP {
   int64_t stride_token;
   int64_t bt_stride;
   int64_t num_blocks;
+  int n_seqs;
   int hn;
-  int group;  // query heads per KV head
-  int nsub;   // query sub-groups per KV head (ceil(group / GT))
+  int group;        // query heads per KV head
+  int nsub;         // query sub-groups per KV head (ceil(group / GT))
+  int pairs_per_seq;  // gn * nsub
   int max_ctx;
-  int part_tokens;
-  int n_parts;
+  int n_waves;      // waves in the main kernel's grid
+  int min_chunk;    // smallest chunk, in tiles
   float scale_log2e;
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
+constexpr int kPlanThreads = 256;
 
-// One WAVE owns one split-K partition of one (sequence, KV head): the waves
-// of a workgroup never synchronise with each other, so a wave that finishes
-// (or has no tokens) retires on its own and the CU always has other waves'
-// loads in flight.  NW only sets how many partitions share a workgroup slot.
+__device__ __forceinline__ int seq_blocks(const DecodeKP &p, int seq, int bs) {
+  int ctx = p.context_lens[seq];
+  ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
+  return ctx > 0 ? (ctx + bs - 1) / bs : 0;
+}
+
+// Tiles per wave: equal shares of the N tiles, never below min_chunk.
+__device__ __forceinline__ int64_t chunk_tiles(const DecodeKP &p, int64_t n_tiles) {
+  int64_t c = (n_tiles + p.n_waves - 1) / p.n_waves;
+  return c < p.min_chunk ? p.min_chunk : c;
+}
+
+// Plan: cum_blocks[s] = sum of block counts of sequences < s.  One workgroup.
+template <int BS>
+__global__ __launch_bounds__(kPlanThreads) void paged_decode_plan_kernel(const DecodeKP p) {
+  __shared__ int32_t s_scan[kPlanThreads];
+  int32_t carry = 0;
+  for (int base = 0; base < p.n_seqs; base += kPlanThreads) {
+    const int s = base + threadIdx.x;
+    const int32_t mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
+    s_scan[threadIdx.x] = mine;
+    __syncthreads();
+    for (int off = 1; off < kPlanThreads; off <<= 1) {
+      const int32_t add = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
+      __syncthreads();
+      s_scan[threadIdx.x] += add;
+      __syncthreads();
+    }
+    if (s < p.n_seqs) p.cum_blocks[s + 1] = carry + s_scan[threadIdx.x];
+    carry += s_scan[kPlanThreads - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) p.cum_blocks[0] = 0;
+}
+
 #ifndef IC_DECODE_NW
 #define IC_DECODE_NW 4
 #endif
-#ifdef IC_DECODE_WAVES_PER_EU
-#define IC_DECODE_OCC __attribute__((amdgpu_waves_per_eu(IC_DECODE_WAVES_PER_EU)))
-#else
-#define IC_DECODE_OCC
-#endif
 
 template <class E, int HD, int GT, int BS, int NW>
-__global__ __launch_bounds__(NW *kWave) IC_DECODE_OCC void paged_decode_kernel(const DecodeKP p) {
+__global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int EPL = E::EPL;
   constexpr int ES = sizeof(T);
   constexpr int LPR = HD / EPL;     // lanes sharing one token row
   constexpr int RPL = kWave / LPR;  // token rows per load instruction
-  constexpr int NLD = BS / RPL;     // load instructions per (block, head) tile
+  constexpr int NLD = BS / RPL;     // load instructions per tile
   static_assert(HD % EPL == 0 && kWave % LPR == 0 && BS % RPL == 0, "tile shape");
+
+  __shared__ __attribute__((aligned(16))) float s_acc[NW][RPL][GT][HD];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int part = blockIdx.x * NW + wave;
-  const int kvh = blockIdx.y / p.nsub;
-  const int sub = blockIdx.y - kvh * p.nsub;
-  const int seq = blockIdx.z;
-
-  int ctx = p.context_lens[seq];
-  ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
-  const int tok_begin = part * p.part_tokens;
-  if (tok_begin >= ctx) return;
-  const int tok_end = (tok_begin + p.part_tokens < ctx) ? tok_begin + p.part_tokens : ctx;
-  const int blk_begin = tok_begin / BS;
-  const int nblk = (tok_end - tok_begin + BS - 1) / BS;  // <= 64 (checked on the host)
-  const int n_parts_seq = (ctx + p.part_tokens - 1) / p.part_tokens;
-
   const int col = lane % LPR;
   const int rowg = lane / LPR;
-  const int head0 = kvh * p.group + sub * GT;  // first query head of this wave
-  const int heads_here = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
 
-  // Lane i keeps the pool block of the partition's i-th block; the loop reads
-  // it back as a wave-uniform scalar (v_readlane), so tile addresses are SALU
-  // work and the table never sits on the load path again.
-  int32_t my_block = 0;
-  if (lane < nblk) {
-    my_block = p.block_tables[seq * p.bt_stride + blk_begin + lane];
-    // A corrupt table entry must not become an out-of-pool address.
-    my_block = my_block < 0 ? 0 : my_block;
-    my_block = (int64_t)my_block >= p.num_blocks ? (int32_t)(p.num_blocks - 1) : my_block;
+  // ---- this wave's chunk of the batch-wide tile sequence ----------------------
+  const int64_t n_tiles = (int64_t)p.cum_blocks[p.n_seqs] * p.pairs_per_seq;
+  const int64_t chunk = chunk_tiles(p, n_tiles);
+  const int64_t wid = (int64_t)blockIdx.x * NW + wave;
+  const int64_t t0 = wid * chunk;
+  if (t0 >= n_tiles) return;
+  int64_t remaining = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;
+
+  // Sequence holding tile t0: the number of sequences that end at or before it.
+  int seq;
+  {
+    int cnt = 0;
+    for (int i = lane; i < p.n_seqs; i += kWave)
+      cnt += ((int64_t)p.cum_blocks[i + 1] * p.pairs_per_seq <= t0) ? 1 : 0;
+    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, kWave);
+    seq = __builtin_amdgcn_readfirstlane(cnt);
   }
-
-  Vec16 qreg[GT];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    qreg[g] = Vec16{{0u, 0u, 0u, 0u}};
-    if (g < heads_here)
-      qreg[g] = load16(p.q + (seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + col * EPL) * ES);
+  int cum = p.cum_blocks[seq];
+  int nb = p.cum_blocks[seq + 1] - cum;  // blocks of this sequence (> 0 by construction)
+  int pair_in_seq, blk;
+  {
+    const int64_t r = t0 - (int64_t)cum * p.pairs_per_seq;
+    pair_in_seq = (int)(r / nb);
+    blk = (int)(r - (int64_t)pair_in_seq * nb);
   }
 
   uint32_t lane_off[NLD];
@@ -132,214 +163,290 @@ __global__ __launch_bounds__(NW *kWave) IC_DECODE_OCC void paged_decode_kernel(c
   for (int i = 0; i < NLD; ++i)
     lane_off[i] = (uint32_t)(((i * RPL + rowg) * p.stride_token + col * EPL) * ES);
 
-  float m[GT], l[GT], acc[GT][EPL];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    m[g] = kNegInf;
-    l[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
-  }
+  while (remaining > 0 && seq < p.n_seqs) {
+    // ---- one segment: blocks [blk, blk_end) of pair (seq, pair_in_seq) --------
+    const int blk_end = (nb - blk < remaining) ? nb : blk + (int)remaining;
+    const int kvh = pair_in_seq / p.nsub;
+    const int sub = pair_in_seq - kvh * p.nsub;
+    const int head0 = kvh * p.group + sub * GT;
+    const int heads_here = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+    int ctx = p.context_lens[seq];
+    ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
 
-  auto issue = [&](int j, Vec16 *kk, Vec16 *vv) {
-    const int64_t phys = __builtin_amdgcn_readlane(my_block, j);
-    const int64_t tile = (phys * p.stride_block + kvh * p.stride_head) * ES;
-    const char *kb = p.k_pool + tile;
-    const char *vb = p.v_pool + tile;
+    Vec16 qreg[GT];
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) kk[i] = load16(kb + lane_off[i]);
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) vv[i] = load16(vb + lane_off[i]);
-    // Keep the loads ahead of the arithmetic that follows in program order:
-    // the scheduler would otherwise sink them below the current tile's work
-    // and shorten the prefetch distance.
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  // `last` marks the partition's final tile, the only one that can be partly
-  // filled; every other tile skips the validity test.
-  auto consume = [&](int j, Vec16 *kk, Vec16 *vv, bool last) {
-    const int tok0 = tok_begin + j * BS;
-    float s[GT][NLD];
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-#pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        float d = E::dot(kk[i], qreg[g], 0.f);
-        s[g][i] = group_sum<LPR>(d) * p.scale_log2e;
-      }
+    for (int g = 0; g < GT; ++g) {
+      qreg[g] = Vec16{{0u, 0u, 0u, 0u}};
+      if (g < heads_here)
+        qreg[g] = load16(p.q + (seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + col * EPL) * ES);
     }
-    if (last && tok0 + BS > tok_end) {  // partly filled block: hide the unused slots
+
+    float m[GT], l[GT], acc[GT][EPL];
 #pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        if (tok0 + i * RPL + rowg >= tok_end) {
+    for (int g = 0; g < GT; ++g) {
+      m[g] = kNegInf;
+      l[g] = 0.f;
 #pragma unroll
-          for (int g = 0; g < GT; ++g) s[g][i] = kNegInf;
-          vv[i] = Vec16{{0u, 0u, 0u, 0u}};
+      for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
+    }
+
+    // Walk the segment in windows of up to 64 blocks (one table entry per lane).
+    for (int win = blk; win < blk_end; win += kWave) {
+      const int nwin = (blk_end - win < kWave) ? blk_end - win : kWave;
+      int32_t my_block = 0;
+      if (lane < nwin) {
+        my_block = p.block_tables[seq * p.bt_stride + win + lane];
+        // A corrupt table entry must not become an out-of-pool address.
+        my_block = my_block < 0 ? 0 : my_block;
+        my_block = (int64_t)my_block >= p.num_blocks ? (int32_t)(p.num_blocks - 1) : my_block;
+      }
+
+      auto issue = [&](int j, Vec16 *kk, Vec16 *vv) {
+        const int64_t phys = __builtin_amdgcn_readlane(my_block, j);
+        const int64_t tile = (phys * p.stride_block + kvh * p.stride_head) * ES;
+        const char *kb = p.k_pool + tile;
+        const char *vb = p.v_pool + tile;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) kk[i] = load16(kb + lane_off[i]);
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) vv[i] = load16(vb + lane_off[i]);
+        // Keep the loads ahead of the arithmetic that follows in program
+        // order: the scheduler would otherwise sink them below the current
+        // tile's work and shorten the prefetch distance.
+        __builtin_amdgcn_sched_barrier(0);
+      };
+
+      // `tail` marks a tile that may be the sequence's last, partly filled
+      // block; every other tile skips the validity test.
+      auto consume = [&](int j, Vec16 *kk, Vec16 *vv, bool tail) {
+        const int tok0 = (win + j) * BS;
+        float s[GT][NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            float d = E::dot(kk[i], qreg[g], 0.f);
+            s[g][i] = group_sum<LPR>(d) * p.scale_log2e;
+          }
         }
+        if (tail && tok0 + BS > ctx) {  // hide the unused slots of the last block
+#pragma unroll
+          for (int i = 0; i < NLD; ++i) {
+            if (tok0 + i * RPL + rowg >= ctx) {
+#pragma unroll
+              for (int g = 0; g < GT; ++g) s[g][i] = kNegInf;
+              vv[i] = Vec16{{0u, 0u, 0u, 0u}};
+            }
+          }
+        }
+        float vf[NLD][EPL];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) E::widen(vv[i], vf[i]);
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          float mx = m[g];
+#pragma unroll
+          for (int i = 0; i < NLD; ++i) mx = fmaxf(mx, s[g][i]);
+          const float ms = (mx == kNegInf) ? 0.f : mx;
+          const float alpha = __builtin_amdgcn_exp2f(m[g] - ms);
+          float pr[NLD];
+          float ps = 0.f;
+#pragma unroll
+          for (int i = 0; i < NLD; ++i) {
+            pr[i] = __builtin_amdgcn_exp2f(s[g][i] - ms);
+            ps += pr[i];
+          }
+          l[g] = l[g] * alpha + ps;
+          m[g] = mx;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            float a = acc[g][e] * alpha;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) a = __builtin_fmaf(pr[i], vf[i][e], a);
+            acc[g][e] = a;
+          }
+        }
+      };
+
+      // The steady-state loop issues the next tile's loads unconditionally, so
+      // the wait before a tile is consumed covers that tile only and the
+      // prefetch stays in flight behind it.
+      Vec16 ka[NLD], va[NLD], kb[NLD], vb[NLD];
+      int j = 0;
+      issue(0, ka, va);
+      for (; j + 2 < nwin; j += 2) {
+        issue(j + 1, kb, vb);
+        consume(j, ka, va, false);
+        issue(j + 2, ka, va);
+        consume(j + 1, kb, vb, false);
+      }
+      if (j + 2 == nwin) {
+        issue(j + 1, kb, vb);
+        consume(j, ka, va, false);
+        consume(j + 1, kb, vb, true);
+      } else {
+        consume(j, ka, va, true);
       }
     }
-    float vf[NLD][EPL];
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) E::widen(vv[i], vf[i]);
+
+    // ---- merge the RPL row groups of this wave (log-sum-exp combine) ---------
+    float lsum[GT], mall[GT];
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
       float mx = m[g];
+      if (RPL >= 2) mx = fmaxf(mx, __shfl_xor(mx, LPR, kWave));
+      if (RPL >= 4) mx = fmaxf(mx, __shfl_xor(mx, 2 * LPR, kWave));
+      if (RPL >= 8) mx = fmaxf(mx, __shfl_xor(mx, 4 * LPR, kWave));
+      const float w = (m[g] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx);
+      float ls = l[g] * w;
+      if (RPL >= 2) ls += __shfl_xor(ls, LPR, kWave);
+      if (RPL >= 4) ls += __shfl_xor(ls, 2 * LPR, kWave);
+      if (RPL >= 8) ls += __shfl_xor(ls, 4 * LPR, kWave);
+      lsum[g] = ls;
+      mall[g] = mx;
 #pragma unroll
-      for (int i = 0; i < NLD; ++i) mx = fmaxf(mx, s[g][i]);
-      const float ms = (mx == kNegInf) ? 0.f : mx;
-      const float alpha = __builtin_amdgcn_exp2f(m[g] - ms);
-      float pr[NLD];
-      float ps = 0.f;
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        pr[i] = __builtin_amdgcn_exp2f(s[g][i] - ms);
-        ps += pr[i];
-      }
-      l[g] = l[g] * alpha + ps;
-      m[g] = mx;
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        float a = acc[g][e] * alpha;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) a = __builtin_fmaf(pr[i], vf[i][e], a);
-        acc[g][e] = a;
+      for (int e = 0; e < EPL; e += 4) {
+        float4 v4 = make_float4(acc[g][e] * w, acc[g][e + 1] * w, acc[g][e + 2] * w, acc[g][e + 3] * w);
+        *reinterpret_cast<float4 *>(&s_acc[wave][rowg][g][col * EPL + e]) = v4;
       }
     }
-  };
+    // Only this wave reads what it wrote: a wave-level fence is enough.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool whole_pair = (blk == 0 && blk_end == nb);
+    const int64_t partial = wid + (int64_t)seq * p.pairs_per_seq + pair_in_seq;
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (g >= heads_here) break;
+      const int h = head0 + g;
+#pragma unroll
+      for (int d = lane; d < HD; d += kWave) {
+        float a = 0.f;
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) a += s_acc[wave][r][g][d];
+        if (whole_pair)
+          reinterpret_cast<T *>(p.out)[seq * p.out_stride_seq + (int64_t)h * HD + d] =
+              E::narrow(a / lsum[g]);
+        else
+          p.part_acc[(partial * GT + g) * HD + d] = a;
+      }
+      if (!whole_pair && lane == 0) {
+        p.part_ml[(partial * GT + g) * 2] = mall[g];
+        p.part_ml[(partial * GT + g) * 2 + 1] = lsum[g];
+      }
+    }
+    // The slab is reused by the next segment.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 
-  {
-    // Two register tiles in ping-pong.  The steady-state loop issues the next
-    // tile's loads unconditionally, so the wait before a tile is consumed
-    // covers that tile only and the prefetch stays in flight behind it.
-    Vec16 ka[NLD], va[NLD], kb[NLD], vb[NLD];
-    int j = 0;
-    issue(0, ka, va);
-    for (; j + 2 < nblk; j += 2) {
-      issue(j + 1, kb, vb);
-      consume(j, ka, va, false);
-      issue(j + 2, ka, va);
-      consume(j + 1, kb, vb, false);
-    }
-    if (j + 2 == nblk) {
-      issue(j + 1, kb, vb);
-      consume(j, ka, va, false);
-      consume(j + 1, kb, vb, true);
-    } else {
-      consume(j, ka, va, true);
-    }
-  }
-
-  // ---- merge the RPL row groups of this wave (log-sum-exp combine) -----------
-  __shared__ __attribute__((aligned(16))) float s_acc[NW][RPL][GT][HD];
-  float lsum[GT], mall[GT];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    float mx = m[g];
-    if (RPL >= 2) mx = fmaxf(mx, __shfl_xor(mx, LPR, kWave));
-    if (RPL >= 4) mx = fmaxf(mx, __shfl_xor(mx, 2 * LPR, kWave));
-    if (RPL >= 8) mx = fmaxf(mx, __shfl_xor(mx, 4 * LPR, kWave));
-    const float w = (m[g] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx);
-    float ls = l[g] * w;
-    if (RPL >= 2) ls += __shfl_xor(ls, LPR, kWave);
-    if (RPL >= 4) ls += __shfl_xor(ls, 2 * LPR, kWave);
-    if (RPL >= 8) ls += __shfl_xor(ls, 4 * LPR, kWave);
-    lsum[g] = ls;
-    mall[g] = mx;
-#pragma unroll
-    for (int e = 0; e < EPL; e += 4) {
-      float4 v4 = make_float4(acc[g][e] * w, acc[g][e + 1] * w, acc[g][e + 2] * w, acc[g][e + 3] * w);
-      *reinterpret_cast<float4 *>(&s_acc[wave][rowg][g][col * EPL + e]) = v4;
-    }
-  }
-  // Only this wave reads what it wrote: a wave-level LDS fence is enough.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    if (g >= heads_here) break;
-    const int h = head0 + g;
-    const int64_t slot = ((int64_t)seq * p.hn + h) * p.n_parts + part;
-#pragma unroll
-    for (int d = lane; d < HD; d += kWave) {
-      float a = 0.f;
-#pragma unroll
-      for (int r = 0; r < RPL; ++r) a += s_acc[wave][r][g][d];
-      if (n_parts_seq == 1)
-        reinterpret_cast<T *>(p.out)[seq * p.out_stride_seq + (int64_t)h * HD + d] = E::narrow(a / lsum[g]);
-      else
-        p.part_acc[slot * HD + d] = a;
-    }
-    if (n_parts_seq != 1 && lane == 0) {
-      p.part_ml[slot * 2] = mall[g];
-      p.part_ml[slot * 2 + 1] = lsum[g];
+    // ---- next pair ------------------------------------------------------------
+    remaining -= blk_end - blk;
+    blk = 0;
+    if (++pair_in_seq == p.pairs_per_seq) {
+      pair_in_seq = 0;
+      do {
+        ++seq;
+        if (seq >= p.n_seqs) break;
+        nb = p.cum_blocks[seq + 1] - p.cum_blocks[seq];
+      } while (nb == 0);
     }
   }
 }
 
 // Combine the split-K partials of one (sequence, query head).
-// grid = (hn, n_seqs), HD threads.  Traffic is n_parts*(hd+2)*4 bytes per
-// head, three orders of magnitude below the K/V stream.
-template <class E, int HD>
+// grid = (hn, n_seqs), HD threads.  A pair's tiles are a contiguous run of the
+// batch-wide sequence, so the waves that touched it are
+// first_tile / chunk .. last_tile / chunk and their partial ids follow.
+// Traffic is (hd+2)*4 bytes per partial, three orders of magnitude below the
+// K/V stream.
+template <class E, int HD, int GT>
 __global__ __launch_bounds__(HD) void paged_decode_reduce_kernel(const DecodeKP p) {
   using T = typename E::type;
   const int h = blockIdx.x;
   const int seq = blockIdx.y;
   const int d = threadIdx.x;
-  int ctx = p.context_lens[seq];
-  ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
   T *o = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)h * HD + d;
-  if (ctx <= 0) {
+  const int cum = p.cum_blocks[seq];
+  const int nb = p.cum_blocks[seq + 1] - cum;
+  if (nb == 0) {
     *o = E::narrow(0.f);
     return;
   }
-  const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
-  if (np == 1) return;  // finished by the main kernel
-  const int64_t slot0 = ((int64_t)seq * p.hn + h) * p.n_parts;
+  const int kvh = h / p.group;
+  const int gi = h - kvh * p.group;
+  const int sub = gi / GT;
+  const int g = gi - sub * GT;
+  const int pair_in_seq = kvh * p.nsub + sub;
+  const int64_t n_tiles = (int64_t)p.cum_blocks[p.n_seqs] * p.pairs_per_seq;
+  const int64_t chunk = chunk_tiles(p, n_tiles);
+  const int64_t first = (int64_t)cum * p.pairs_per_seq + (int64_t)pair_in_seq * nb;
+  const int64_t w0 = first / chunk;
+  const int64_t w1 = (first + nb - 1) / chunk;
+  if (w0 == w1) return;  // one wave covered the whole pair and wrote the row
+  const int64_t base = (int64_t)seq * p.pairs_per_seq + pair_in_seq;
   float mx = kNegInf;
-  for (int i = 0; i < np; ++i) mx = fmaxf(mx, p.part_ml[(slot0 + i) * 2]);
+  for (int64_t w = w0; w <= w1; ++w) mx = fmaxf(mx, p.part_ml[((w + base) * GT + g) * 2]);
   float lsum = 0.f, a = 0.f;
-  for (int i = 0; i < np; ++i) {
-    const float w = __builtin_amdgcn_exp2f(p.part_ml[(slot0 + i) * 2] - mx);
-    lsum = __builtin_fmaf(p.part_ml[(slot0 + i) * 2 + 1], w, lsum);
-    a = __builtin_fmaf(p.part_acc[(slot0 + i) * HD + d], w, a);
+  for (int64_t w = w0; w <= w1; ++w) {
+    const int64_t slot = (w + base) * GT + g;
+    const float wt = __builtin_amdgcn_exp2f(p.part_ml[slot * 2] - mx);
+    lsum = __builtin_fmaf(p.part_ml[slot * 2 + 1], wt, lsum);
+    a = __builtin_fmaf(p.part_acc[slot * HD + d], wt, a);
   }
   *o = E::narrow(a / lsum);
 }
 
+// Waves of the main kernel that one GPU holds at once, per kernel variant.
+template <class E, int HD, int GT, int BS, int NW>
+int resident_workgroups() {
+  static const int per_cu = [] {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_kernel<E, HD, GT, BS, NW>,
+                                                     NW * kWave, 0) != hipSuccess || n < 1)
+      n = 1;
+    return n;
+  }();
+  return per_cu * device_cu_count();
+}
+
 template <class E, int HD, int GT>
-int launch_typed(const DecodeKP &kp, int gn, int n_seqs, hipStream_t stream) {
+int launch_typed(DecodeKP &kp, hipStream_t stream) {
   constexpr int BS = 16;
   constexpr int NW = IC_DECODE_NW;
-  dim3 grid((kp.n_parts + NW - 1) / NW, gn * kp.nsub, n_seqs);
-  hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), grid, dim3(NW * kWave), 0, stream, kp);
-  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD>), dim3(kp.hn, n_seqs), dim3(HD), 0, stream, kp);
+  int wgs = resident_workgroups<E, HD, GT, BS, NW>();
+  if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
+  kp.n_waves = wgs * NW;
+  hipLaunchKernelGGL((paged_decode_plan_kernel<BS>), dim3(1), dim3(kPlanThreads), 0, stream, kp);
+  hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
+  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD, GT>), dim3(kp.hn, kp.n_seqs), dim3(HD), 0,
+                     stream, kp);
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;
 }
 
 template <class E, int HD>
-int launch_group(DecodeKP &kp, int gn, int n_seqs, hipStream_t stream) {
+int launch_group(DecodeKP &kp, int gn, hipStream_t stream) {
   const int G = kp.group;
-  const int gt = G <= 8 ? G : 8;
+  const int gt = decode_heads_per_wave(G);
   kp.nsub = (G + gt - 1) / gt;
+  kp.pairs_per_seq = gn * kp.nsub;
   switch (gt) {
-    case 1: return launch_typed<E, HD, 1>(kp, gn, n_seqs, stream);
-    case 2: return launch_typed<E, HD, 2>(kp, gn, n_seqs, stream);
-    case 3: return launch_typed<E, HD, 3>(kp, gn, n_seqs, stream);
-    case 4: return launch_typed<E, HD, 4>(kp, gn, n_seqs, stream);
-    case 5: return launch_typed<E, HD, 5>(kp, gn, n_seqs, stream);
-    case 6: return launch_typed<E, HD, 6>(kp, gn, n_seqs, stream);
-    case 7: return launch_typed<E, HD, 7>(kp, gn, n_seqs, stream);
-    default: return launch_typed<E, HD, 8>(kp, gn, n_seqs, stream);
+    case 1: return launch_typed<E, HD, 1>(kp, stream);
+    case 2: return launch_typed<E, HD, 2>(kp, stream);
+    case 3: return launch_typed<E, HD, 3>(kp, stream);
+    case 4: return launch_typed<E, HD, 4>(kp, stream);
+    case 5: return launch_typed<E, HD, 5>(kp, stream);
+    case 6: return launch_typed<E, HD, 6>(kp, stream);
+    case 7: return launch_typed<E, HD, 7>(kp, stream);
+    default: return launch_typed<E, HD, 8>(kp, stream);
   }
 }
 
 template <class E>
-int launch_hd(DecodeKP &kp, int hd, int gn, int n_seqs, hipStream_t stream) {
+int launch_hd(DecodeKP &kp, int hd, int gn, hipStream_t stream) {
   switch (hd) {
-    case 64: return launch_group<E, 64>(kp, gn, n_seqs, stream);
-    case 128: return launch_group<E, 128>(kp, gn, n_seqs, stream);
+    case 64: return launch_group<E, 64>(kp, gn, stream);
+    case 128: return launch_group<E, 128>(kp, gn, stream);
     default: return IC_ERR_UNSUPPORTED;
   }
 }
@@ -355,6 +462,7 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.block_tables = a.block_tables;
   kp.context_lens = a.context_lens;
   kp.out = (char *)a.out;
+  kp.cum_blocks = a.cum_blocks;
   kp.part_ml = a.part_ml;
   kp.part_acc = a.part_acc;
   kp.q_stride_seq = a.q_stride_seq;
@@ -364,17 +472,19 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.stride_token = a.pool.stride_token;
   kp.bt_stride = a.block_table_stride;
   kp.num_blocks = a.pool.num_blocks;
+  kp.n_seqs = a.n_seqs;
   kp.hn = a.hn;
   kp.group = a.hn / a.gn;
   kp.nsub = 1;
+  kp.pairs_per_seq = a.gn;
   kp.max_ctx = a.max_context_len;
-  kp.part_tokens = a.part_tokens;
-  kp.n_parts = a.n_parts;
+  kp.n_waves = 0;
+  kp.min_chunk = a.min_chunk_tokens / a.pool.block_size;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
   switch (a.dtype) {
-    case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.gn, a.n_seqs, stream);
-    case IC_DTYPE_F16: return launch_hd<F16>(kp, a.hd, a.gn, a.n_seqs, stream);
-    case IC_DTYPE_F32: return launch_hd<F32>(kp, a.hd, a.gn, a.n_seqs, stream);
+    case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.gn, stream);
+    case IC_DTYPE_F16: return launch_hd<F16>(kp, a.hd, a.gn, stream);
+    case IC_DTYPE_F32: return launch_hd<F32>(kp, a.hd, a.gn, stream);
     default: return IC_ERR_UNSUPPORTED;
   }
 }

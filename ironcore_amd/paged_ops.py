@@ -87,11 +87,12 @@ def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_pool: torch.Tensor, v_
 def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                  block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
                  scale: float | None = None, out: torch.Tensor | None = None,
-                 part_tokens: int = 0) -> torch.Tensor:
+                 min_chunk_tokens: int = 0) -> torch.Tensor:
     """One query token per sequence.  ``query`` ``[b, hn, hd]`` -> ``[b, hn*hd]``.
 
-    ``max_context_len`` is a host-side upper bound on ``context_lens`` (it
-    sizes the split-K grid without a device synchronisation)."""
+    ``max_context_len`` is a host-side upper bound on ``context_lens`` (no
+    device synchronisation is needed to launch).  ``min_chunk_tokens`` is the
+    smallest split-K share (0 = library default)."""
     lib = _lib.load()
     dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens)
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
@@ -118,14 +119,14 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
         raise ValueError("out must be [b, hn*hd] in the query dtype with contiguous rows")
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
-    need = lib.ic_paged_decode_workspace_bytes(b, hn, hd, max(max_context_len, 1), part_tokens)
+    need = lib.ic_paged_decode_workspace_bytes(b, hn, gn, hd)
     ws = _workspace.get(dev, need)
     with torch.cuda.device(dev):
         rc = lib.ic_paged_decode(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
                                  k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
                                  block_tables.data_ptr(), block_tables.stride(0),
                                  context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
-                                 float(scale), part_tokens, ws.data_ptr(), ws.numel(),
+                                 float(scale), min_chunk_tokens, ws.data_ptr(), ws.numel(),
                                  _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
     _lib.check("ic_paged_decode", rc)
     return out
