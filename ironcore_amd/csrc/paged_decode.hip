@@ -13,20 +13,23 @@
 //    byte is fetched once per KV head, not once per query head.  (G > 8 is
 //    cut into sub-groups of <= 8 heads, each its own pair.)
 //  * Split-K by equal shares: the tiles of the whole batch form one sequence
-//    (pair-major, block-minor); a plan kernel prefix-sums the per-sequence
-//    block counts, and every resident WAVE takes one contiguous chunk of
+//    (pair-major, block-minor); every resident WAVE prefix-sums the
+//    per-sequence block counts and takes one contiguous chunk of
 //    ceil(N / waves) tiles.  A chunk may start and end inside a pair and may
 //    span several pairs; each (wave, pair) segment yields one partial.  All
 //    waves carry the same load whatever the spread of context lengths, the
 //    grid is exactly the number of waves the GPU holds at once, and waves
 //    never synchronise with each other.
-//  * Block ids of up to 64 blocks sit one per lane and are read back as
-//    wave-uniform scalars (v_readlane), so tile addresses are SALU work.
+//  * At the start of its chunk a wave gathers the byte offsets of its next
+//    256 tiles from the block table, one per lane and slot; the loop reads
+//    them back as wave-uniform scalars (v_readlane), so the table is off the
+//    load path and tile addresses are SALU work.
 //  * One tile is block_size*hd contiguous elements per K and per V; each lane
 //    fetches 16 bytes per load, so one load instruction covers 1 KiB of
 //    consecutive bytes (64/LPR token rows, LPR = lanes per row).  Two
 //    register tiles in ping-pong: the next tile's loads are in flight while
-//    the current one is consumed.
+//    the current one is consumed, across pair boundaries too; the next
+//    pair's query is prefetched a segment ahead.
 //  * q.k: v_dot2 on the packed pairs, then a DPP butterfly over the LPR lanes
 //    that share a row.  Online softmax per lane group; p*v accumulates into
 //    EPL fp32 registers per query head with no cross-lane traffic.
@@ -74,7 +77,6 @@ struct DecodeKP {
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
-constexpr int kPlanThreads = 256;
 
 __device__ __forceinline__ int seq_blocks(const DecodeKP &p, int seq, int bs) {
   int ctx = p.context_lens[seq];
@@ -88,32 +90,45 @@ __device__ __forceinline__ int64_t chunk_tiles(const DecodeKP &p, int64_t n_tile
   return c < p.min_chunk ? p.min_chunk : c;
 }
 
-// Plan: cum_blocks[s] = sum of block counts of sequences < s.  One workgroup.
-template <int BS>
-__global__ __launch_bounds__(kPlanThreads) void paged_decode_plan_kernel(const DecodeKP p) {
-  __shared__ int32_t s_scan[kPlanThreads];
-  int32_t carry = 0;
-  for (int base = 0; base < p.n_seqs; base += kPlanThreads) {
-    const int s = base + threadIdx.x;
-    const int32_t mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
-    s_scan[threadIdx.x] = mine;
-    __syncthreads();
-    for (int off = 1; off < kPlanThreads; off <<= 1) {
-      const int32_t add = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
-      __syncthreads();
-      s_scan[threadIdx.x] += add;
-      __syncthreads();
-    }
-    if (s < p.n_seqs) p.cum_blocks[s + 1] = carry + s_scan[threadIdx.x];
-    carry += s_scan[kPlanThreads - 1];
-    __syncthreads();
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int up = __shfl_up(v, off, kWave);
+    v += lane >= off ? up : 0;
   }
-  if (threadIdx.x == 0) p.cum_blocks[0] = 0;
+  return v;
 }
 
 #ifndef IC_DECODE_NW
 #define IC_DECODE_NW 4
 #endif
+
+// Position in the batch-wide tile sequence: block `blk` of pair
+// (seq, pair) whose sequence has `nb` blocks.  Wave-uniform.
+struct TileCursor {
+  int seq;
+  int pair;
+  int blk;
+  int nb;
+};
+
+template <int BS>
+__device__ __forceinline__ void next_pair(const DecodeKP &p, TileCursor &c) {
+  c.blk = 0;
+  if (++c.pair == p.pairs_per_seq) {
+    c.pair = 0;
+    do {
+      ++c.seq;
+      if (c.seq >= p.n_seqs) {  // past the last tile: never dereferenced
+        c.seq = p.n_seqs;
+        c.nb = 0x7fffffff;
+        return;
+      }
+      c.nb = seq_blocks(p, c.seq, BS);
+    } while (c.nb == 0);
+  }
+}
 
 template <class E, int HD, int GT, int BS, int NW>
 __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP p) {
@@ -123,6 +138,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   constexpr int LPR = HD / EPL;     // lanes sharing one token row
   constexpr int RPL = kWave / LPR;  // token rows per load instruction
   constexpr int NLD = BS / RPL;     // load instructions per tile
+  constexpr int SW = 4;             // tile offsets held per lane: a window is 64*SW tiles
   static_assert(HD % EPL == 0 && kWave % LPR == 0 && BS % RPL == 0, "tile shape");
 
   __shared__ __attribute__((aligned(16))) float s_acc[NW][RPL][GT][HD];
@@ -133,163 +149,94 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   const int rowg = lane / LPR;
 
   // ---- this wave's chunk of the batch-wide tile sequence ----------------------
-  const int64_t n_tiles = (int64_t)p.cum_blocks[p.n_seqs] * p.pairs_per_seq;
-  const int64_t chunk = chunk_tiles(p, n_tiles);
+  // Every wave prefix-sums the per-sequence block counts itself (64 sequences
+  // per step, one per lane): first for the total, which fixes the chunk size,
+  // then again to find the sequence that holds its first tile.  Wave 0 also
+  // leaves the prefix sums in the workspace for the reduce kernel.
   const int64_t wid = (int64_t)blockIdx.x * NW + wave;
+  int64_t total_blocks = 0;
+  for (int base = 0; base < p.n_seqs; base += kWave) {
+    const int s = base + lane;
+    const int mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
+    const int incl = wave_inclusive_scan(mine, lane);
+    if (wid == 0 && s < p.n_seqs) p.cum_blocks[s + 1] = (int32_t)(total_blocks + incl);
+    total_blocks += __builtin_amdgcn_readlane(incl, kWave - 1);
+  }
+  if (wid == 0 && lane == 0) p.cum_blocks[0] = 0;
+  const int64_t n_tiles = total_blocks * p.pairs_per_seq;
+  const int64_t chunk = chunk_tiles(p, n_tiles);
   const int64_t t0 = wid * chunk;
   if (t0 >= n_tiles) return;
-  int64_t remaining = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;
+  int64_t left = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;  // tiles not yet consumed
 
-  // Sequence holding tile t0: the number of sequences that end at or before it.
-  int seq;
+  TileCursor c;
   {
-    int cnt = 0;
-    for (int i = lane; i < p.n_seqs; i += kWave)
-      cnt += ((int64_t)p.cum_blocks[i + 1] * p.pairs_per_seq <= t0) ? 1 : 0;
-    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, kWave);
-    seq = __builtin_amdgcn_readfirstlane(cnt);
-  }
-  int cum = p.cum_blocks[seq];
-  int nb = p.cum_blocks[seq + 1] - cum;  // blocks of this sequence (> 0 by construction)
-  int pair_in_seq, blk;
-  {
+    int64_t before = 0;  // blocks of the sequences scanned so far
+    c.seq = p.n_seqs;
+    c.nb = 1;
+    int cum = 0;
+    for (int base = 0; base < p.n_seqs; base += kWave) {
+      const int s = base + lane;
+      const int mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
+      const int incl = wave_inclusive_scan(mine, lane);
+      // first sequence whose tiles end after t0
+      const uint64_t hit = __ballot((before + incl) * p.pairs_per_seq > t0);
+      if (hit != 0) {
+        const int ln = __builtin_ctzll(hit);
+        c.seq = base + ln;
+        c.nb = __builtin_amdgcn_readlane(mine, ln);
+        cum = (int)(before + __builtin_amdgcn_readlane(incl, ln)) - c.nb;
+        break;
+      }
+      before += __builtin_amdgcn_readlane(incl, kWave - 1);
+    }
     const int64_t r = t0 - (int64_t)cum * p.pairs_per_seq;
-    pair_in_seq = (int)(r / nb);
-    blk = (int)(r - (int64_t)pair_in_seq * nb);
+    c.pair = (int)(r / c.nb);
+    c.blk = (int)(r - (int64_t)c.pair * c.nb);
   }
+  TileCursor walk = c;  // gathers tile addresses ahead of the arithmetic
+  TileCursor peek = c;  // the segment after the current one (its q is prefetched)
+  next_pair<BS>(p, peek);
+  int seg_blk0 = c.blk;
 
   uint32_t lane_off[NLD];
 #pragma unroll
   for (int i = 0; i < NLD; ++i)
     lane_off[i] = (uint32_t)(((i * RPL + rowg) * p.stride_token + col * EPL) * ES);
 
-  while (remaining > 0 && seq < p.n_seqs) {
-    // ---- one segment: blocks [blk, blk_end) of pair (seq, pair_in_seq) --------
-    const int blk_end = (nb - blk < remaining) ? nb : blk + (int)remaining;
-    const int kvh = pair_in_seq / p.nsub;
-    const int sub = pair_in_seq - kvh * p.nsub;
+  auto load_q = [&](const TileCursor &tc, Vec16 *qq) {
+    const int kvh = tc.pair / p.nsub;
+    const int sub = tc.pair - kvh * p.nsub;
     const int head0 = kvh * p.group + sub * GT;
-    const int heads_here = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
-    int ctx = p.context_lens[seq];
-    ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
-
-    Vec16 qreg[GT];
+    const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
-      qreg[g] = Vec16{{0u, 0u, 0u, 0u}};
-      if (g < heads_here)
-        qreg[g] = load16(p.q + (seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + col * EPL) * ES);
+      qq[g] = Vec16{{0u, 0u, 0u, 0u}};
+      if (g < heads && tc.seq < p.n_seqs)
+        qq[g] = load16(p.q + (tc.seq * p.q_stride_seq + (int64_t)(head0 + g) * HD + col * EPL) * ES);
     }
+  };
+  Vec16 qreg[GT], qnext[GT];
+  load_q(c, qreg);
+  load_q(peek, qnext);
 
-    float m[GT], l[GT], acc[GT][EPL];
+  float m[GT], l[GT], acc[GT][EPL];
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      m[g] = kNegInf;
-      l[g] = 0.f;
+  for (int g = 0; g < GT; ++g) {
+    m[g] = kNegInf;
+    l[g] = 0.f;
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
-    }
+    for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
+  }
 
-    // Walk the segment in windows of up to 64 blocks (one table entry per lane).
-    for (int win = blk; win < blk_end; win += kWave) {
-      const int nwin = (blk_end - win < kWave) ? blk_end - win : kWave;
-      int32_t my_block = 0;
-      if (lane < nwin) {
-        my_block = p.block_tables[seq * p.bt_stride + win + lane];
-        // A corrupt table entry must not become an out-of-pool address.
-        my_block = my_block < 0 ? 0 : my_block;
-        my_block = (int64_t)my_block >= p.num_blocks ? (int32_t)(p.num_blocks - 1) : my_block;
-      }
-
-      auto issue = [&](int j, Vec16 *kk, Vec16 *vv) {
-        const int64_t phys = __builtin_amdgcn_readlane(my_block, j);
-        const int64_t tile = (phys * p.stride_block + kvh * p.stride_head) * ES;
-        const char *kb = p.k_pool + tile;
-        const char *vb = p.v_pool + tile;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) kk[i] = load16(kb + lane_off[i]);
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) vv[i] = load16(vb + lane_off[i]);
-        // Keep the loads ahead of the arithmetic that follows in program
-        // order: the scheduler would otherwise sink them below the current
-        // tile's work and shorten the prefetch distance.
-        __builtin_amdgcn_sched_barrier(0);
-      };
-
-      // `tail` marks a tile that may be the sequence's last, partly filled
-      // block; every other tile skips the validity test.
-      auto consume = [&](int j, Vec16 *kk, Vec16 *vv, bool tail) {
-        const int tok0 = (win + j) * BS;
-        float s[GT][NLD];
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-#pragma unroll
-          for (int g = 0; g < GT; ++g) {
-            float d = E::dot(kk[i], qreg[g], 0.f);
-            s[g][i] = group_sum<LPR>(d) * p.scale_log2e;
-          }
-        }
-        if (tail && tok0 + BS > ctx) {  // hide the unused slots of the last block
-#pragma unroll
-          for (int i = 0; i < NLD; ++i) {
-            if (tok0 + i * RPL + rowg >= ctx) {
-#pragma unroll
-              for (int g = 0; g < GT; ++g) s[g][i] = kNegInf;
-              vv[i] = Vec16{{0u, 0u, 0u, 0u}};
-            }
-          }
-        }
-        float vf[NLD][EPL];
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) E::widen(vv[i], vf[i]);
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
-          float mx = m[g];
-#pragma unroll
-          for (int i = 0; i < NLD; ++i) mx = fmaxf(mx, s[g][i]);
-          const float ms = (mx == kNegInf) ? 0.f : mx;
-          const float alpha = __builtin_amdgcn_exp2f(m[g] - ms);
-          float pr[NLD];
-          float ps = 0.f;
-#pragma unroll
-          for (int i = 0; i < NLD; ++i) {
-            pr[i] = __builtin_amdgcn_exp2f(s[g][i] - ms);
-            ps += pr[i];
-          }
-          l[g] = l[g] * alpha + ps;
-          m[g] = mx;
-#pragma unroll
-          for (int e = 0; e < EPL; ++e) {
-            float a = acc[g][e] * alpha;
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) a = __builtin_fmaf(pr[i], vf[i][e], a);
-            acc[g][e] = a;
-          }
-        }
-      };
-
-      // The steady-state loop issues the next tile's loads unconditionally, so
-      // the wait before a tile is consumed covers that tile only and the
-      // prefetch stays in flight behind it.
-      Vec16 ka[NLD], va[NLD], kb[NLD], vb[NLD];
-      int j = 0;
-      issue(0, ka, va);
-      for (; j + 2 < nwin; j += 2) {
-        issue(j + 1, kb, vb);
-        consume(j, ka, va, false);
-        issue(j + 2, ka, va);
-        consume(j + 1, kb, vb, false);
-      }
-      if (j + 2 == nwin) {
-        issue(j + 1, kb, vb);
-        consume(j, ka, va, false);
-        consume(j + 1, kb, vb, true);
-      } else {
-        consume(j, ka, va, true);
-      }
-    }
-
-    // ---- merge the RPL row groups of this wave (log-sum-exp combine) ---------
+  // End of a segment: merge the RPL row groups of the wave (log-sum-exp)
+  // through the wave's LDS slab, write the output row or a partial, then move
+  // to the next pair.  The next tile's loads are already in flight.
+  auto finish_segment = [&]() {
+    const int kvh = c.pair / p.nsub;
+    const int sub = c.pair - kvh * p.nsub;
+    const int head0 = kvh * p.group + sub * GT;
+    const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
     float lsum[GT], mall[GT];
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
@@ -309,16 +256,20 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
         float4 v4 = make_float4(acc[g][e] * w, acc[g][e + 1] * w, acc[g][e + 2] * w, acc[g][e + 3] * w);
         *reinterpret_cast<float4 *>(&s_acc[wave][rowg][g][col * EPL + e]) = v4;
       }
+      m[g] = kNegInf;
+      l[g] = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
     }
     // Only this wave reads what it wrote: a wave-level fence is enough.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const bool whole_pair = (blk == 0 && blk_end == nb);
-    const int64_t partial = wid + (int64_t)seq * p.pairs_per_seq + pair_in_seq;
+    const bool whole_pair = (seg_blk0 == 0 && c.blk == c.nb);
+    const int64_t partial = wid + (int64_t)c.seq * p.pairs_per_seq + c.pair;
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
-      if (g >= heads_here) break;
+      if (g >= heads) break;
       const int h = head0 + g;
 #pragma unroll
       for (int d = lane; d < HD; d += kWave) {
@@ -326,7 +277,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
 #pragma unroll
         for (int r = 0; r < RPL; ++r) a += s_acc[wave][r][g][d];
         if (whole_pair)
-          reinterpret_cast<T *>(p.out)[seq * p.out_stride_seq + (int64_t)h * HD + d] =
+          reinterpret_cast<T *>(p.out)[c.seq * p.out_stride_seq + (int64_t)h * HD + d] =
               E::narrow(a / lsum[g]);
         else
           p.part_acc[(partial * GT + g) * HD + d] = a;
@@ -339,17 +290,160 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
     // The slab is reused by the next segment.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    if (left > 0) {
+      c = peek;
+      seg_blk0 = 0;
+#pragma unroll
+      for (int g = 0; g < GT; ++g) qreg[g] = qnext[g];
+      next_pair<BS>(p, peek);
+      load_q(peek, qnext);
+    }
+  };
 
-    // ---- next pair ------------------------------------------------------------
-    remaining -= blk_end - blk;
-    blk = 0;
-    if (++pair_in_seq == p.pairs_per_seq) {
-      pair_in_seq = 0;
-      do {
-        ++seq;
-        if (seq >= p.n_seqs) break;
-        nb = p.cum_blocks[seq + 1] - p.cum_blocks[seq];
-      } while (nb == 0);
+  // One tile of arithmetic on the registers (kk, vv), for the tile at cursor c.
+  auto consume = [&](Vec16 *kk, Vec16 *vv) {
+    float s[GT][NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        float d = E::dot(kk[i], qreg[g], 0.f);
+        s[g][i] = group_sum<LPR>(d) * p.scale_log2e;
+      }
+    }
+    if (c.blk == c.nb - 1) {  // the sequence's last block may be partly filled
+      int ctx = p.context_lens[c.seq];
+      ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
+      const int tok0 = c.blk * BS;
+      if (tok0 + BS > ctx) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+          if (tok0 + i * RPL + rowg >= ctx) {
+#pragma unroll
+            for (int g = 0; g < GT; ++g) s[g][i] = kNegInf;
+            vv[i] = Vec16{{0u, 0u, 0u, 0u}};
+          }
+        }
+      }
+    }
+    float vf[NLD][EPL];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) E::widen(vv[i], vf[i]);
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      float mx = m[g];
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) mx = fmaxf(mx, s[g][i]);
+      const float ms = (mx == kNegInf) ? 0.f : mx;
+      const float alpha = __builtin_amdgcn_exp2f(m[g] - ms);
+      float pr[NLD];
+      float ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        pr[i] = __builtin_amdgcn_exp2f(s[g][i] - ms);
+        ps += pr[i];
+      }
+      l[g] = l[g] * alpha + ps;
+      m[g] = mx;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        float a = acc[g][e] * alpha;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) a = __builtin_fmaf(pr[i], vf[i][e], a);
+        acc[g][e] = a;
+      }
+    }
+    ++c.blk;
+    --left;
+    if (c.blk == c.nb || left == 0) finish_segment();
+  };
+
+  while (left > 0) {
+    // ---- window: byte offsets of the next n_win tiles, one per lane and slot ---
+    const int n_win = left < kWave * SW ? (int)left : kWave * SW;
+    int64_t row_idx[SW];
+    int32_t kv_of[SW];
+#pragma unroll
+    for (int r = 0; r < SW; ++r) {
+      row_idx[r] = 0;
+      kv_of[r] = 0;
+    }
+    for (int pos = 0; pos < n_win;) {  // wave-uniform walk over the window's segments
+      const int cnt = (walk.nb - walk.blk < n_win - pos) ? walk.nb - walk.blk : n_win - pos;
+      const int kvh = walk.pair / p.nsub;
+      const int64_t base = (int64_t)walk.seq * p.bt_stride + walk.blk - pos;
+#pragma unroll
+      for (int r = 0; r < SW; ++r) {
+        const int lp = r * kWave + lane;
+        const bool in = lp >= pos && lp < pos + cnt;
+        row_idx[r] = in ? base + lp : row_idx[r];
+        kv_of[r] = in ? kvh : kv_of[r];
+      }
+      pos += cnt;
+      walk.blk += cnt;
+      if (walk.blk == walk.nb) next_pair<BS>(p, walk);
+    }
+    uint32_t off_lo[SW], off_hi[SW];
+#pragma unroll
+    for (int r = 0; r < SW; ++r) {
+      int64_t phys = 0;
+      if (r * kWave + lane < n_win) phys = p.block_tables[row_idx[r]];
+      // A corrupt table entry must not become an out-of-pool address.
+      phys = phys < 0 ? 0 : phys;
+      phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
+      const int64_t off = (phys * p.stride_block + (int64_t)kv_of[r] * p.stride_head) * ES;
+      off_lo[r] = (uint32_t)off;
+      off_hi[r] = (uint32_t)(off >> 32);
+    }
+
+    auto issue = [&](int i, Vec16 *kk, Vec16 *vv) {
+      const int ln = i & (kWave - 1);
+      uint32_t lo, hi;
+      if (i < kWave) {
+        lo = __builtin_amdgcn_readlane(off_lo[0], ln);
+        hi = __builtin_amdgcn_readlane(off_hi[0], ln);
+      } else if (i < 2 * kWave) {
+        lo = __builtin_amdgcn_readlane(off_lo[1], ln);
+        hi = __builtin_amdgcn_readlane(off_hi[1], ln);
+      } else if (i < 3 * kWave) {
+        lo = __builtin_amdgcn_readlane(off_lo[2], ln);
+        hi = __builtin_amdgcn_readlane(off_hi[2], ln);
+      } else {
+        lo = __builtin_amdgcn_readlane(off_lo[3], ln);
+        hi = __builtin_amdgcn_readlane(off_hi[3], ln);
+      }
+      const int64_t tile = (int64_t)(((uint64_t)hi << 32) | lo);
+      const char *kb = p.k_pool + tile;
+      const char *vb = p.v_pool + tile;
+#pragma unroll
+      for (int q4 = 0; q4 < NLD; ++q4) kk[q4] = load16(kb + lane_off[q4]);
+#pragma unroll
+      for (int q4 = 0; q4 < NLD; ++q4) vv[q4] = load16(vb + lane_off[q4]);
+      // Keep the loads ahead of the arithmetic that follows in program order:
+      // the scheduler would otherwise sink them below the current tile's work
+      // and shorten the prefetch distance.
+      __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Two register tiles in ping-pong.  The steady-state loop issues the next
+    // tile's loads unconditionally, so the wait before a tile is consumed
+    // covers that tile only and the prefetch stays in flight behind it,
+    // across pair boundaries too.
+    Vec16 ka[NLD], va[NLD], kb[NLD], vb[NLD];
+    int i = 0;
+    issue(0, ka, va);
+    for (; i + 2 < n_win; i += 2) {
+      issue(i + 1, kb, vb);
+      consume(ka, va);
+      issue(i + 2, ka, va);
+      consume(kb, vb);
+    }
+    if (i + 2 == n_win) {
+      issue(i + 1, kb, vb);
+      consume(ka, va);
+      consume(kb, vb);
+    } else {
+      consume(ka, va);
     }
   }
 }
@@ -417,7 +511,6 @@ int launch_typed(DecodeKP &kp, hipStream_t stream) {
   int wgs = resident_workgroups<E, HD, GT, BS, NW>();
   if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
   kp.n_waves = wgs * NW;
-  hipLaunchKernelGGL((paged_decode_plan_kernel<BS>), dim3(1), dim3(kPlanThreads), 0, stream, kp);
   hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
   hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD, GT>), dim3(kp.hn, kp.n_seqs), dim3(HD), 0,
                      stream, kp);
