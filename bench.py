@@ -39,6 +39,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) so a counter run can be scaled")
     return ap.parse_args()
 
 
@@ -92,6 +94,14 @@ def main():
     parity = (out[:n_chk].float().cpu() - ref.float()).abs().max().item()
     if not parity <= 2e-2:
         sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- timed region ---------------------------------------------------------
     for i in range(args.warmup):
