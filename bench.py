@@ -1,20 +1,27 @@
 #!/usr/bin/env python3
-"""Headline benchmark: paged decode, Llama-7B layer shape, batch 64.
+"""Benchmarks of the paged-attention hot path on one MI355X.
 
+Default (the headline line): paged decode, Llama-7B layer shape, batch 64.
 One step = one pass of the decode hot path over one batch for one transformer
-layer: KV append of the 64 new K/V rows, then paged attention of the 64 query
-tokens against the block KV cache (32 q heads, 32 kv heads, head_dim 128,
-bf16, block 16, context lengths uniform in [512, 4096], randomly permuted
-block tables, q/K/V ~ N(0,1)).  Several layers' pools are resident and the
-steps rotate over them, as a decoder's layers do, so no step re-reads the
+layer: KV append of the new K/V rows (one per sequence), then paged attention
+of the query tokens against the block KV cache (32 q heads, 32 kv heads,
+head_dim 128, bf16, block 16, context lengths uniform in [512, 4096], randomly
+permuted block tables, q/K/V ~ N(0,1)).  Several layers' pools are resident
+and the steps rotate over them, as a decoder's layers do, so no step re-reads
 bytes the previous one left in cache.
 
-Prints ONE JSON line.  `value` is achieved HBM GB/s of the whole step
-(algorithmic bytes / wall time per step); decode tokens/s are reported beside
-it.  `roofline` describes the decode call (main kernel + its split-K reduce)
-timed with events on the launch stream; `cpu_baseline` is the CPU oracle (the
-reference's dense attention arithmetic driven through the block table) timed
-on the host cores on a bounded sample of the same workload.
+`--workload llama70b | grpo` run the GQA and the shared-prefix decode shapes
+the same way; `--workload prefill` runs chunked prefill + KV append (16
+sequences, cached prefix uniform in [0, 4096], 512 new tokens each) and
+reports TFLOP/s against the dense bf16 MFMA peak.
+
+Prints ONE JSON line.  For decode `value` is achieved HBM GB/s of the whole
+step (algorithmic bytes / wall time per step), with decode tokens/s beside it;
+`roofline` describes the dominant call (decode: main kernel + its split-K
+reduce; prefill: the MFMA kernel) timed with events on the launch stream;
+`cpu_baseline` is the CPU oracle (the reference's dense attention arithmetic
+driven through the block table) timed on the host cores on a bounded sample
+of the same workload.
 """
 from __future__ import annotations
 
@@ -25,7 +32,13 @@ import statistics
 import sys
 import time
 
-HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, vendor figure
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
+
+# HBM bytes per launch of the decode main kernel on the default workload
+# (llama7b, seed 0), from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
+# 1 GiB device copy in the same process (profiles/paged_decode_llama7b_bs64_hbm_counters.md).
+MEASURED_TRAFFIC = {("llama7b", 0): 2466400000}
 
 
 def parse():
@@ -35,7 +48,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=4, help="resident layer pools the steps rotate over")
     ap.add_argument("--min-chunk-tokens", type=int, default=0, help="smallest split-K share (0 = library default)")
-    ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo"])
+    ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo", "prefill"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
     ap.add_argument("--seed", type=int, default=0)
@@ -44,33 +57,55 @@ def parse():
     return ap.parse_args()
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: the paged-attention path is single-GPU "
-                 "(sequences and KV heads shard without communication); run with --gpus 1")
+def cpu_info():
     import torch
+    try:
+        model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
+    except Exception:
+        model = "unknown"
+    return {"cores": torch.get_num_threads(), "host_cpu_count": os.cpu_count(), "cpu_model": model}
+
+
+def copy_calibration(torch, dev):
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
+def time_steps(torch, step, steps, warmup):
+    """Run `warmup` untimed steps, then exactly `steps` timed ones bracketed by
+    synchronisations.  `step(i, ev)` enqueues step i and records the event pair
+    `ev` around its dominant call.  Returns (ms per step by wall clock, list of
+    per-call ms from the events)."""
+    for i in range(warmup):
+        step(i, None)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, ev[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in ev]
+
+
+def bench_decode(args, torch, dev):
     from ironcore_amd import paged_ops, workloads
-
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU (the paged path has no CPU implementation)")
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-
+    from oracle import paged as oracle_paged
     make = {"llama7b": workloads.llama7b_decode, "llama70b": workloads.llama70b_gqa_decode,
             "grpo": workloads.qwen7b_grpo_decode}[args.workload]
     wl = make(device=dev, seed=args.seed)
     b, hn, gn, hd, bs = wl.batch, wl.hn, wl.gn, wl.hd, wl.block_size
-    # one pool pair per resident layer (layer 0 is the workload's own)
-    pools = [(wl.k_pool, wl.v_pool)]
+    pools = [(wl.k_pool, wl.v_pool)]          # one pool pair per resident layer
     for layer in range(1, args.layers):
         g = torch.Generator(device=dev)
         g.manual_seed(args.seed + 100 + layer)
         pools.append(tuple(torch.randn(wl.k_pool.shape, generator=g, device=dev, dtype=torch.float32)
                            .to(wl.k_pool.dtype) for _ in range(2)))
     # the step's new K/V rows go to the slot of each sequence's last token
-    ctx = wl.context_lens.long()
-    last = ctx - 1
+    last = wl.context_lens.long() - 1
     slot_mapping = (wl.block_tables.long().gather(1, (last // bs).unsqueeze(1)).squeeze(1) * bs + last % bs)
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed + 7)
@@ -78,15 +113,18 @@ def main():
     v_new = torch.randn(b, gn, hd, generator=g, device=dev, dtype=torch.float32).to(wl.k_pool.dtype)
     out = torch.empty(b, hn * hd, dtype=wl.query.dtype, device=dev)
 
-    def step(i):
+    def step(i, ev):
         kp, vp = pools[i % len(pools)]
         paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
+        if ev:
+            ev[0].record()
         paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
                                wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens)
+        if ev:
+            ev[1].record()
 
-    # ---- parity gate on the tensors that are about to be timed --------------
-    from oracle import paged as oracle_paged
-    step(0)
+    # parity gate on the tensors that are about to be timed
+    step(0, None)
     torch.cuda.synchronize()
     n_chk = min(b, 6)
     ref = oracle_paged.paged_decode(wl.query[:n_chk].cpu(), pools[0][0].cpu(), pools[0][1].cpu(),
@@ -94,74 +132,47 @@ def main():
     parity = (out[:n_chk].float().cpu() - ref.float()).abs().max().item()
     if not parity <= 2e-2:
         sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
-
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(torch, dev)
 
-    # ---- timed region ---------------------------------------------------------
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        kp, vp = pools[i % len(pools)]
-        paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
-        ev[i][0].record()
-        paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
-                               wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    decode_ms = [a.elapsed_time(c) for a, c in ev]
+    ms_per_step, decode_ms = time_steps(torch, step, args.steps, args.warmup)
     decode_ms_avg = sum(decode_ms) / len(decode_ms)
-
     es = wl.query.element_size()
     decode_bytes = wl.algorithmic_bytes()
     append_bytes = 2 * (2 * b * gn * hd * es) + 8 * b
-    step_bytes = decode_bytes + append_bytes
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    value = (decode_bytes + append_bytes) / (ms_per_step * 1e-3) / 1e9
     achieved = decode_bytes / (decode_ms_avg * 1e-3) / 1e9
-
     result = {
-        "metric": "paged_decode_hbm_gbps",
-        "value": round(value, 1),
-        "unit": "GB/s",
+        "metric": "paged_decode_hbm_gbps", "value": round(value, 1), "unit": "GB/s",
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "decode_tokens_per_s_per_layer": round(b / (ms_per_step * 1e-3), 1),
         "decode_tokens_per_s_32_layers": round(b / (32 * ms_per_step * 1e-3), 1),
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl.name, "batch": b, "q_heads": hn, "kv_heads": gn, "head_dim": hd,
                    "block_size": bs, "sum_context": wl.logical_tokens, "unique_tokens": wl.unique_tokens,
                    "resident_layers": len(pools),
-                   "step": "kv_append(64 rows) + paged_decode, one layer"},
+                   "step": f"kv_append({b} rows) + paged_decode, one layer"},
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.seed)),
                      "kernel": "paged_decode_kernel (+ split-K reduce)",
                      "bytes_per_launch": decode_bytes, "avg_launch_ms": round(decode_ms_avg, 5),
                      "median_launch_ms": round(statistics.median(decode_ms), 5)},
     }
-
+    if wl.logical_tokens != wl.unique_tokens:
+        logical = wl.logical_tokens * wl.kv_bytes_per_token()
+        result["logical_kv_gbps"] = round(logical / (decode_ms_avg * 1e-3) / 1e9, 1)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(wl, pools[0], args.cpu_seconds)
-    print(json.dumps(result))
+        result["cpu_baseline"] = cpu_baseline_decode(wl, pools[0], args.cpu_seconds)
+    return result
 
 
-def cpu_baseline(wl, pool, budget_s):
+def cpu_baseline_decode(wl, pool, budget_s):
     """The CPU oracle on a bounded sample: the first n sequences of the same
-    batch (same block tables, same pools), median of >= 3 repetitions."""
-    import torch
+    batch (same block tables, same pools), median of 3 repetitions."""
     from oracle import paged as oracle_paged
     kp, vp = pool[0].cpu(), pool[1].cpu()
     q, bt, cl = wl.query.cpu(), wl.block_tables.cpu(), wl.context_lens.cpu()
@@ -177,15 +188,98 @@ def cpu_baseline(wl, pool, budget_s):
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
     tokens = int(cl[:n].sum())
-    nbytes = tokens * wl.kv_bytes_per_token()
-    try:
-        model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
-    except Exception:
-        model = "unknown"
-    return {"value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"first {n} of {wl.batch} sequences of the same batch, one layer, "
-            f"median of 3 (after 1 warm-up); {tokens} context tokens",
-            "tokens_per_s_per_layer": round(n / t, 2), "host_cpu_count": os.cpu_count(), "cpu_model": model}
+    return {"value": round(tokens * wl.kv_bytes_per_token() / t / 1e9, 3), "unit": "GB/s", "kind": "port",
+            "sample": f"first {n} of {wl.batch} sequences of the same batch, one layer, "
+                      f"median of 3 (after 1 warm-up); {tokens} context tokens",
+            "tokens_per_s_per_layer": round(n / t, 2), **cpu_info()}
+
+
+def bench_prefill(args, torch, dev):
+    from ironcore_amd import paged_ops, workloads
+    from oracle import paged as oracle_paged
+    wl = workloads.llama7b_chunked_prefill(device=dev, seed=args.seed)
+    out = torch.empty(wl.query.shape[0], wl.hn * wl.hd, dtype=wl.query.dtype, device=dev)
+
+    def step(i, ev):
+        paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)
+        if ev:
+            ev[0].record()
+        paged_ops.paged_prefill(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens,
+                                wl.cu_seqlens_q, wl.max_chunk_len, causal=True, out=out)
+        if ev:
+            ev[1].record()
+
+    # parity gate: the sequence with the shortest prefix, all heads, against the oracle
+    step(0, None)
+    torch.cuda.synchronize()
+    i = min(range(len(wl.prefix_lens)), key=lambda j: wl.prefix_lens[j])
+    lo, hi = int(wl.cu_seqlens_q[i]), int(wl.cu_seqlens_q[i + 1])
+    one = (wl.query[lo:hi].cpu(), wl.k_pool.cpu(), wl.v_pool.cpu(), wl.block_tables[i:i + 1].cpu(),
+           wl.context_lens[i:i + 1].cpu(), torch.tensor([0, hi - lo], dtype=torch.int32))
+    ref = oracle_paged.paged_prefill(*one)
+    parity = (out[lo:hi].float().cpu() - ref.float()).abs().max().item()
+    if not parity <= 2e-2:
+        sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
+    if args.copy_calibration:
+        copy_calibration(torch, dev)
+
+    ms_per_step, call_ms = time_steps(torch, step, args.steps, args.warmup)
+    call_avg = sum(call_ms) / len(call_ms)
+    flops = wl.flops()
+    es = wl.query.element_size()
+    append_bytes = 2 * 2 * wl.k_new.numel() * es
+    tflops = flops / (call_avg * 1e-3) / 1e12
+    n_tok = wl.query.shape[0]
+
+    def append_only(i, ev):
+        if ev:
+            ev[0].record()
+        paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)
+        if ev:
+            ev[1].record()
+    _, app_ms = time_steps(torch, append_only, 50, 5)
+
+    result = {
+        "metric": "paged_prefill_mfma_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "prefill_tokens_per_s_per_layer": round(n_tok / (ms_per_step * 1e-3), 1),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": wl.name, "n_seqs": len(wl.chunk_lens), "chunk": wl.max_chunk_len,
+                   "sum_prefix": sum(wl.prefix_lens), "q_heads": wl.hn, "kv_heads": wl.gn,
+                   "head_dim": wl.hd, "block_size": wl.block_size,
+                   "step": "kv_append(chunk rows) + paged_prefill, one layer"},
+        "parity_max_abs_vs_oracle": parity,
+        "append_hbm_gbps": round(append_bytes / (statistics.mean(app_ms) * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "paged_prefill_kernel", "flops_per_launch": flops,
+                     "avg_launch_ms": round(call_avg, 5), "median_launch_ms": round(statistics.median(call_ms), 5)},
+    }
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        oracle_paged.paged_prefill(*one)
+        t = time.perf_counter() - t0
+        c, pfx = wl.chunk_lens[i], wl.prefix_lens[i]
+        f = 4 * wl.hn * wl.hd * (c * pfx + c * (c + 1) // 2)
+        result["cpu_baseline"] = {"value": round(f / t / 1e12, 4), "unit": "TFLOP/s", "kind": "port",
+                                  "sample": f"one sequence of the batch (prefix {pfx}, chunk {c}), all heads, 1 run",
+                                  **cpu_info()}
+    return result
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the paged-attention path is single-GPU "
+                 "(sequences and KV heads shard without communication); run with --gpus 1")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the paged path has no CPU implementation)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    result = bench_prefill(args, torch, dev) if args.workload == "prefill" else bench_decode(args, torch, dev)
+    print(json.dumps(result))
 
 
 if __name__ == "__main__":

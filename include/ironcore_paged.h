@@ -111,7 +111,8 @@ size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd);
  *                 to it, and block_table_stride must cover it
  *   min_chunk_tokens  the K/V stream of the whole batch is cut into equal
  *                 shares, one per resident wave (split-K); this is the
- *                 smallest share (multiple of block_size), 0 = default
+ *                 smallest share (multiple of 16), 0 = default
+ *   block_size    a multiple of 16 (the kernel loads whole 16-token tiles)
  *   workspace     at least ic_paged_decode_workspace_bytes(...) bytes, 256-byte
  *                 aligned; contents need not be initialised
  * Sequences with context_lens[i] <= 0 produce zeros.

@@ -22,9 +22,9 @@ int check_pool(int64_t sb, int64_t sh, int64_t st, int gn, int hd, int block_siz
   return IC_OK;
 }
 
-int resolve_min_chunk(int min_chunk_tokens, int block_size) {
+int resolve_min_chunk(int min_chunk_tokens) {
   if (min_chunk_tokens == 0) min_chunk_tokens = ic::kDefaultMinChunkTokens;
-  if (min_chunk_tokens < block_size || min_chunk_tokens % block_size != 0) return -1;
+  if (min_chunk_tokens < 16 || min_chunk_tokens % 16 != 0) return -1;
   return min_chunk_tokens;
 }
 
@@ -117,7 +117,7 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
   if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
   if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
   if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
-  const int mc = resolve_min_chunk(min_chunk_tokens, block_size);
+  const int mc = resolve_min_chunk(min_chunk_tokens);
   if (mc < 0) return IC_ERR_BAD_SHAPE;
   const int64_t need_blocks = ((int64_t)max_context_len + block_size - 1) / block_size;
   if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;

@@ -8,8 +8,9 @@
 //
 // HBM-bound streaming kernel (one pass over every visible K and V byte).
 //
-//  * Unit of work: a TILE = one pool block (16 tokens) of one (sequence, KV
-//    head) "pair", for ALL G query heads that share the KV head, so each K/V
+//  * Unit of work: a TILE = 16 consecutive tokens of one (sequence, KV head)
+//    "pair" (one pool block at block size 16, a slice of a longer block
+//    otherwise), for ALL G query heads that share the KV head, so each K/V
 //    byte is fetched once per KV head, not once per query head.  (G > 8 is
 //    cut into sub-groups of <= 8 heads, each its own pair.)
 //  * Split-K by equal shares: the tiles of the whole batch form one sequence
@@ -73,6 +74,7 @@ struct DecodeKP {
   int max_ctx;
   int n_waves;      // waves in the main kernel's grid
   int min_chunk;    // smallest chunk, in tiles
+  int tiles_per_block;  // 16-token tiles in one pool block (1 for block_size 16)
   float scale_log2e;
 };
 
@@ -362,22 +364,31 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
     // ---- window: byte offsets of the next n_win tiles, one per lane and slot ---
     const int n_win = left < kWave * SW ? (int)left : kWave * SW;
     int64_t row_idx[SW];
-    int32_t kv_of[SW];
+    int32_t kv_of[SW], sub_of[SW];
 #pragma unroll
     for (int r = 0; r < SW; ++r) {
       row_idx[r] = 0;
       kv_of[r] = 0;
+      sub_of[r] = 0;
     }
     for (int pos = 0; pos < n_win;) {  // wave-uniform walk over the window's segments
       const int cnt = (walk.nb - walk.blk < n_win - pos) ? walk.nb - walk.blk : n_win - pos;
       const int kvh = walk.pair / p.nsub;
-      const int64_t base = (int64_t)walk.seq * p.bt_stride + walk.blk - pos;
+      const int64_t row = (int64_t)walk.seq * p.bt_stride;
 #pragma unroll
       for (int r = 0; r < SW; ++r) {
         const int lp = r * kWave + lane;
         const bool in = lp >= pos && lp < pos + cnt;
-        row_idx[r] = in ? base + lp : row_idx[r];
+        int tile_in_seq = walk.blk + lp - pos;
+        int sub = 0;
+        if (p.tiles_per_block > 1) {  // pool blocks longer than one tile
+          const int b = tile_in_seq / p.tiles_per_block;
+          sub = tile_in_seq - b * p.tiles_per_block;
+          tile_in_seq = b;
+        }
+        row_idx[r] = in ? row + tile_in_seq : row_idx[r];
         kv_of[r] = in ? kvh : kv_of[r];
+        sub_of[r] = in ? sub : sub_of[r];
       }
       pos += cnt;
       walk.blk += cnt;
@@ -391,7 +402,8 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
       // A corrupt table entry must not become an out-of-pool address.
       phys = phys < 0 ? 0 : phys;
       phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
-      const int64_t off = (phys * p.stride_block + (int64_t)kv_of[r] * p.stride_head) * ES;
+      const int64_t off = (phys * p.stride_block + (int64_t)kv_of[r] * p.stride_head +
+                           (int64_t)sub_of[r] * BS * p.stride_token) * ES;
       off_lo[r] = (uint32_t)off;
       off_hi[r] = (uint32_t)(off >> 32);
     }
@@ -547,7 +559,9 @@ int launch_hd(DecodeKP &kp, int hd, int gn, hipStream_t stream) {
 }  // namespace
 
 int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
-  if (a.pool.block_size != 16) return IC_ERR_UNSUPPORTED;
+  // The kernel loads whole 16-token tiles, so a pool block must hold a whole
+  // number of them (a tile never straddles the end of a block).
+  if (a.pool.block_size % 16 != 0) return IC_ERR_UNSUPPORTED;
   DecodeKP kp;
   kp.q = (const char *)a.q;
   kp.k_pool = (const char *)a.k_pool;
@@ -572,7 +586,8 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.pairs_per_seq = a.gn;
   kp.max_ctx = a.max_context_len;
   kp.n_waves = 0;
-  kp.min_chunk = a.min_chunk_tokens / a.pool.block_size;
+  kp.min_chunk = (a.min_chunk_tokens + 15) / 16;
+  kp.tiles_per_block = a.pool.block_size / 16;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
   switch (a.dtype) {
     case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.gn, stream);

@@ -1,0 +1,300 @@
+"""Generation through the block KV cache: the model-side callers of the
+attention layer and the generate loop.
+
+The reference reaches its attention layer only through
+``LanguageModel.forward`` -> ``TransformerModel`` -> ``TransformerLayer.
+custom_forward`` (ironcore/language_model.py:67-100, ironcore/models/
+transformer.py:77-162) and generates by re-running that forward on the whole
+growing sequence every step (examples/generate_text.py:12-46).  The classes
+below keep that arithmetic and those parameter names, add the two optional
+arguments that carry the KV cache down to ``Attention.forward``, and replace
+the full recompute by prefill + cached decode.  The GEMMs, norms and the
+activation are plain torch calls on the GPU (plumbing around the hot path);
+attention and the KV append are the HIP kernels.
+
+Only what the reference's GPT-2-shaped configuration exercises is built:
+pre/post-LN LayerNorm, learned absolute positions, GELU/ReLU/SiLU MLP, tied or
+untied output embedding.  RoPE is left out on purpose: the reference's rotary
+module indexes its angles by batch index (ironcore/layers/positional_embedding/
+rotary.py:53-64), which a KV-cached path cannot reproduce meaningfully.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .kv_cache import PagedKVCache
+from .layers.attention import Attention
+from .layers.module import BaseModule, get_model_dtype
+
+
+class Linear(BaseModule):
+    """``y = x @ W + b`` with the weight stored ``[in, out]`` as the reference's
+    parallel linears do at tensor-parallel size 1
+    (ironcore/parallel/tensor_parallel/layers.py:41,194-204,250-263)."""
+
+    def __init__(self, config, input_size: int, output_size: int, bias: bool):
+        super().__init__(config)
+        self.weight = nn.Parameter(torch.empty(input_size, output_size))
+        self.bias = nn.Parameter(torch.empty(output_size)) if bias else None
+
+    def forward(self, x):
+        y = torch.matmul(x, self.weight)
+        return y + self.bias if self.bias is not None else y
+
+
+class LayerNorm(BaseModule):
+    """ironcore/layers/layernorm/fused_layer_norm.py:20-28 (wraps nn.LayerNorm)."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.layernorm = nn.LayerNorm(config.model.d_model, eps=config.model.ln_eps,
+                                      bias=not config.model.no_bias)
+
+    def forward(self, x):
+        return self.layernorm(x)
+
+
+def get_activation(name: str) -> nn.Module:
+    """ironcore/layers/activations/activations.py:45-60 (non-GLU variants)."""
+    if name == "relu":
+        return nn.ReLU()
+    if name == "gelu":
+        return nn.GELU()
+    if name == "silu":
+        return nn.SiLU()
+    raise NotImplementedError(f"activation {name!r} is not part of the generation path")
+
+
+class MLP(BaseModule):
+    """ironcore/layers/mlp.py:19-54 without dropout (inference)."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        bias = not config.model.no_bias
+        self.activation = get_activation(config.model.activation_type)
+        self.up_proj = Linear(config, config.model.d_model, config.model.d_ffn, bias)
+        self.down_proj = Linear(config, config.model.d_ffn, config.model.d_model, bias)
+
+    def forward(self, x):
+        return self.down_proj(self.activation(self.up_proj(x)))
+
+
+class TransformerLayer(BaseModule):
+    """ironcore/models/transformer.py:23-135.  The new K/V rows exist right
+    after the projections (transformer.py:88-98): that is where they enter the
+    cache, inside ``self_attention``."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        m = config.model
+        bias = not m.no_bias
+        self.head_dimension = m.d_model // m.num_attention_heads
+        self.num_local_attention_heads = m.num_attention_heads // config.trainer.tensor_model_parallel_size
+        self.num_local_attention_groups = m.num_attention_groups // config.trainer.tensor_model_parallel_size
+        self.linear_q = Linear(config, m.d_model, m.head_dim * m.num_attention_heads, bias)
+        self.linear_kv = Linear(config, m.d_model, m.head_dim * m.num_attention_groups * 2, bias)
+        self.attn_output = Linear(config, m.head_dim * m.num_attention_heads, m.d_model, bias)
+        self.input_layernorm = LayerNorm(config)
+        self.self_attention = Attention(config)
+        self.post_attn_layernorm = LayerNorm(config)
+        self.mlp = MLP(config)
+
+    def forward(self, hidden_states, attention_mask, rotary_pos_emb=None, *, kv_cache=None,
+                attn_metadata=None):
+        if rotary_pos_emb is not None:
+            raise NotImplementedError("rotary embeddings are not part of the generation path")
+        b, s, _ = hidden_states.shape
+        norm_output = self.input_layernorm(hidden_states)
+        query = self.linear_q(norm_output)
+        key, value = torch.chunk(self.linear_kv(norm_output), 2, dim=-1)
+        query = query.view(b, s, self.num_local_attention_heads, self.head_dimension)
+        key = key.view(b, s, self.num_local_attention_groups, self.head_dimension)
+        value = value.view(b, s, self.num_local_attention_groups, self.head_dimension)
+        attention_output = self.self_attention(query, key, value, attention_mask, kv_cache=kv_cache,
+                                               attn_metadata=attn_metadata)
+        attention_output = self.attn_output(attention_output)
+        residual = norm_output if self.config.model.post_ln else hidden_states
+        norm_input = residual + attention_output
+        norm_output = self.post_attn_layernorm(norm_input)
+        mlp_output = self.mlp(norm_output)
+        residual = norm_output if self.config.model.post_ln else norm_input
+        return residual + mlp_output
+
+
+class TransformerModel(BaseModule):
+    """ironcore/models/transformer.py:138-162."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.layers = nn.ModuleList([TransformerLayer(config) for _ in range(config.model.num_layers)])
+
+    def forward(self, hidden_states, attention_mask, rotary_pos_emb=None, *, kv_cache: Optional[PagedKVCache] = None,
+                attn_metadata=None):
+        for index, layer in enumerate(self.layers):
+            hidden_states = layer(hidden_states, attention_mask, rotary_pos_emb,
+                                  kv_cache=None if kv_cache is None else kv_cache.layer(index),
+                                  attn_metadata=attn_metadata)
+        return hidden_states
+
+
+class LanguageModelEmbedding(BaseModule):
+    """ironcore/layers/embedding.py:9-50 (word + learned absolute position)."""
+
+    def __init__(self, config, padded_vocab_size: int):
+        super().__init__(config)
+        if config.model.positional_embedding.type != "absolute":
+            raise NotImplementedError("only learned absolute positions are part of the generation path")
+        self.word_embeddings = nn.Embedding(padded_vocab_size, config.model.d_model)
+        self.position_embedding = nn.Embedding(config.model.max_seq_len, config.model.d_model)
+
+    def forward(self, input_ids, position_ids):
+        return self.word_embeddings(input_ids) + self.position_embedding(position_ids)
+
+
+def padded_vocab(vocab_size: int, unit: int = 128) -> int:
+    """The reference pads the vocabulary to a multiple of 128 and zeroes the
+    padded rows (ironcore/tokenizer/tokenizer.py:70-75,
+    ironcore/parallel/tensor_parallel/layers.py:116-118)."""
+    return (vocab_size + unit - 1) // unit * unit
+
+
+class LanguageModel(BaseModule):
+    """ironcore/language_model.py:21-100,203-227, inference only (labels=None):
+    returns logits ``[b, s, padded_vocab]``.
+
+    ``forward(input_ids)`` is the reference's full causal pass.
+    ``forward(input_ids, kv_cache=cache, seq_ids=ids)`` treats ``input_ids`` as
+    the NEW tokens of sequences that already live in ``cache`` (prefill when
+    they are empty, one token per step afterwards)."""
+
+    def __init__(self, config, vocab_size: int = 50257):
+        super().__init__(config)
+        self.vocab_size = vocab_size
+        self.padded_vocab_size = padded_vocab(vocab_size, config.trainer.vocab_padding_unit)
+        self.embedding = LanguageModelEmbedding(config, self.padded_vocab_size)
+        self.model = TransformerModel(config)
+        self.output_layernorm = LayerNorm(config)
+        if config.model.untie_embed:
+            self.output_layer = Linear(config, config.model.d_model, self.padded_vocab_size, bias=False)
+        self.init_weights()
+
+    def init_weights(self):
+        """ironcore/layers/module.py:43-76 at tensor-parallel size 1: biases 0,
+        norm scales 1, everything else N(0, init_std), residual projections
+        N(0, init_std / sqrt(2 * layers)); padded vocabulary rows zeroed."""
+        std = self.init_std
+        with torch.no_grad():
+            for name, param in self.named_parameters():
+                if "bias" in name:
+                    param.zero_()
+                elif "norm" in name:
+                    param.fill_(1.0)
+                elif name.endswith("output.weight") or name.endswith("down_proj.weight"):
+                    param.normal_(mean=0.0, std=std / math.sqrt(2 * self.config.model.num_layers))
+                else:
+                    param.normal_(mean=0.0, std=std)
+            self.embedding.word_embeddings.weight[self.vocab_size:].zero_()
+
+    def forward(self, input_ids, labels=None, *, kv_cache: Optional[PagedKVCache] = None,
+                seq_ids: Optional[Sequence[int]] = None):
+        if labels is not None:
+            raise NotImplementedError("loss computation is a training feature")
+        b, s = input_ids.shape
+        dev = input_ids.device
+        if kv_cache is None:
+            attention_mask = torch.tril(torch.ones(s, s, device=dev)).view(1, 1, s, s) > 0.5
+            position_ids = torch.arange(s, device=dev).unsqueeze(0).expand(b, s)
+            meta = None
+        else:
+            if seq_ids is None or len(seq_ids) != b:
+                raise ValueError("one cache sequence id per batch row")
+            past = [kv_cache.length(sid) for sid in seq_ids]
+            meta = kv_cache.prepare(seq_ids, s)
+            attention_mask = None
+            position_ids = (torch.tensor(past, device=dev).unsqueeze(1) + torch.arange(s, device=dev).unsqueeze(0))
+        x = self.embedding(input_ids, position_ids)
+        x = self.model(x, attention_mask, None, kv_cache=kv_cache, attn_metadata=meta)
+        x = self.output_layernorm(x)
+        if self.config.model.untie_embed:
+            return torch.matmul(x, self.output_layer.weight)
+        return torch.matmul(x, self.embedding.word_embeddings.weight.transpose(0, 1))
+
+
+def sample_next(logits: torch.Tensor, temperature: float = 0.0, top_k: int = 0,
+                generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """Next token from last-position logits ``[b, vocab]``.  ``temperature == 0``
+    is greedy argmax; otherwise temperature and top-k sampling exactly as
+    examples/generate_text.py:28-37 does them (scale, drop everything below the
+    k-th logit, softmax, multinomial)."""
+    if temperature == 0.0:
+        return logits.argmax(dim=-1, keepdim=True)
+    logits = logits / temperature
+    if top_k > 0:
+        kth = torch.topk(logits, top_k)[0][..., -1, None]
+        logits = logits.masked_fill(logits < kth, float("-inf"))
+    probs = torch.softmax(logits, dim=-1)
+    return torch.multinomial(probs, num_samples=1, generator=generator)
+
+
+@torch.no_grad()
+def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int, *,
+             block_size: int = 16, temperature: float = 0.0, top_k: int = 0,
+             eos_token_id: Optional[int] = None, generator: Optional[torch.Generator] = None,
+             kv_cache: Optional[PagedKVCache] = None, return_margins: bool = False):
+    """Batched generation through the block KV cache: one prefill pass over the
+    prompts, then one cached decode step per new token.  Equal-length prompts
+    ``[b, s]``.  Returns ``[b, s + n]`` token ids (and, on request, the per-step
+    top-1/top-2 logit margins ``[b, n]``).  The next token is always chosen
+    from the last position's logits, as examples/generate_text.py:27-28 does."""
+    model.eval()
+    b, s = input_ids.shape
+    cfg = model.config.model
+    if s + max_new_tokens > cfg.max_seq_len:
+        raise ValueError("prompt + new tokens exceed the position table")
+    own_cache = kv_cache is None
+    if own_cache:
+        per_seq = (s + max_new_tokens + block_size - 1) // block_size
+        kv_cache = PagedKVCache(cfg.num_layers, b * per_seq, block_size, cfg.num_attention_groups,
+                                cfg.d_model // cfg.num_attention_heads,
+                                next(model.parameters()).dtype, input_ids.device)
+    seq_ids = [kv_cache.add_sequence() for _ in range(b)]
+    tokens = input_ids
+    margins = []
+    finished = torch.zeros(b, dtype=torch.bool, device=input_ids.device)
+    step_input = input_ids
+    for _ in range(max_new_tokens):
+        logits = model(step_input, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
+        if return_margins:
+            top2 = torch.topk(logits.float(), 2, dim=-1)[0]
+            margins.append(top2[:, 0] - top2[:, 1])
+        nxt = sample_next(logits, temperature, top_k, generator)
+        if eos_token_id is not None:
+            nxt = torch.where(finished.unsqueeze(1), torch.full_like(nxt, eos_token_id), nxt)
+            finished |= nxt.squeeze(1) == eos_token_id
+        tokens = torch.cat([tokens, nxt], dim=1)
+        step_input = nxt
+        if eos_token_id is not None and bool(finished.all()):
+            break
+    if own_cache:
+        for sid in seq_ids:
+            kv_cache.free_sequence(sid)
+    if return_margins:
+        return tokens, torch.stack(margins, dim=1)
+    return tokens
+
+
+@torch.no_grad()
+def generate_full_recompute(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int):
+    """The reference's loop (examples/generate_text.py:24-40) with greedy
+    selection: the whole sequence goes through the model at every step."""
+    model.eval()
+    tokens = input_ids
+    for _ in range(max_new_tokens):
+        logits = model(tokens)[:, -1, :]
+        tokens = torch.cat([tokens, logits.argmax(dim=-1, keepdim=True)], dim=1)
+    return tokens

@@ -1,0 +1,185 @@
+"""Block KV cache: pools, block allocator with prefix sharing, batch metadata.
+
+The reference has no KV cache (its only generation loop recomputes the whole
+sequence every step, examples/generate_text.py:24-40), so this interface is
+defined here.  One ``PagedKVCache`` serves all layers of a model:
+
+* per layer a K pool and a V pool ``[num_blocks, gn, block_size, hd]``
+  (native layout of the kernels: one (block, KV head) tile is contiguous);
+* one block table per sequence, shared by all layers (layer ``l`` of a
+  sequence uses the same block ids in layer ``l``'s pools);
+* a host-side allocator with reference counts, so sequences forked from a
+  common prompt (GRPO groups) alias the prompt's full blocks and copy only the
+  partly filled last block.
+
+Everything the kernels need per step comes from :meth:`PagedKVCache.prepare`,
+which advances the sequences by the step's new tokens and returns a
+``PagedAttentionMetadata`` (block tables, context lengths, slot mapping).  The
+allocator state lives on the host; ``prepare`` uploads small int tensors and
+never reads anything back from the GPU.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Iterable, Sequence
+
+import torch
+
+from .layers.attention import PagedAttentionMetadata
+
+
+class OutOfBlocks(RuntimeError):
+    """The pool has no free block left."""
+
+
+class BlockAllocator:
+    """Free list + reference counts over ``num_blocks`` pool blocks."""
+
+    def __init__(self, num_blocks: int):
+        self.num_blocks = num_blocks
+        self._free = list(range(num_blocks - 1, -1, -1))
+        self._refs = [0] * num_blocks
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> int:
+        if not self._free:
+            raise OutOfBlocks(f"all {self.num_blocks} KV blocks are in use")
+        blk = self._free.pop()
+        self._refs[blk] = 1
+        return blk
+
+    def share(self, blk: int) -> int:
+        if self._refs[blk] <= 0:
+            raise ValueError(f"block {blk} is not allocated")
+        self._refs[blk] += 1
+        return blk
+
+    def release(self, blk: int) -> None:
+        if self._refs[blk] <= 0:
+            raise ValueError(f"block {blk} is not allocated")
+        self._refs[blk] -= 1
+        if self._refs[blk] == 0:
+            self._free.append(blk)
+
+    def ref_count(self, blk: int) -> int:
+        return self._refs[blk]
+
+
+@dataclass
+class _Sequence:
+    blocks: list = field(default_factory=list)
+    length: int = 0
+
+
+class PagedKVCache:
+    """Pools for ``num_layers`` layers plus the sequences that live in them."""
+
+    def __init__(self, num_layers: int, num_blocks: int, block_size: int, num_kv_heads: int,
+                 head_dim: int, dtype: torch.dtype, device):
+        if block_size % 16 != 0:
+            raise ValueError("block_size must be a multiple of 16 (the kernels walk 16-token tiles)")
+        self.num_layers = num_layers
+        self.num_blocks = num_blocks
+        self.block_size = block_size
+        self.device = torch.device(device)
+        shape = (num_layers, num_blocks, num_kv_heads, block_size, head_dim)
+        self.k_pools = torch.zeros(shape, dtype=dtype, device=self.device)
+        self.v_pools = torch.zeros(shape, dtype=dtype, device=self.device)
+        self.allocator = BlockAllocator(num_blocks)
+        self._seqs: dict[int, _Sequence] = {}
+        self._next_id = 0
+
+    # ---- pools -----------------------------------------------------------------
+    def layer(self, index: int):
+        """(k_pool, v_pool) of one layer, the ``kv_cache`` argument of
+        ``Attention.forward``."""
+        return self.k_pools[index], self.v_pools[index]
+
+    # ---- sequences ---------------------------------------------------------------
+    def add_sequence(self) -> int:
+        sid = self._next_id
+        self._next_id += 1
+        self._seqs[sid] = _Sequence()
+        return sid
+
+    def length(self, sid: int) -> int:
+        return self._seqs[sid].length
+
+    def blocks(self, sid: int) -> list:
+        return list(self._seqs[sid].blocks)
+
+    def free_sequence(self, sid: int) -> None:
+        for blk in self._seqs.pop(sid).blocks:
+            self.allocator.release(blk)
+
+    def fork(self, sid: int) -> int:
+        """New sequence with the same content: full blocks are aliased
+        (reference count up), a partly filled last block is copied so that the
+        two sequences can append independently."""
+        src = self._seqs[sid]
+        child = _Sequence(length=src.length)
+        full = src.length // self.block_size
+        for blk in src.blocks[:full]:
+            child.blocks.append(self.allocator.share(blk))
+        if src.length % self.block_size:
+            new = self.allocator.allocate()
+            old = src.blocks[full]
+            self.k_pools[:, new].copy_(self.k_pools[:, old])
+            self.v_pools[:, new].copy_(self.v_pools[:, old])
+            child.blocks.append(new)
+        cid = self._next_id
+        self._next_id += 1
+        self._seqs[cid] = child
+        return cid
+
+    def _slot_for_append(self, seq: _Sequence) -> int:
+        """Slot of the next token; allocates a block at block boundaries and
+        un-shares an aliased block before it is written (copy on write)."""
+        bs = self.block_size
+        idx, off = divmod(seq.length, bs)
+        if idx == len(seq.blocks):
+            seq.blocks.append(self.allocator.allocate())
+        blk = seq.blocks[idx]
+        if self.allocator.ref_count(blk) > 1:
+            new = self.allocator.allocate()
+            self.k_pools[:, new].copy_(self.k_pools[:, blk])
+            self.v_pools[:, new].copy_(self.v_pools[:, blk])
+            self.allocator.release(blk)
+            seq.blocks[idx] = blk = new
+        seq.length += 1
+        return blk * bs + off
+
+    # ---- per-step metadata -----------------------------------------------------------
+    def prepare(self, seq_ids: Sequence[int], new_tokens: int | Iterable[int]) -> PagedAttentionMetadata:
+        """Advance each sequence by its number of new tokens (one int for all,
+        or one per sequence, padded to the longest with slot -1) and build the
+        step's metadata.  The new K/V rows must then be passed through
+        ``Attention.forward(..., kv_cache=cache.layer(l), attn_metadata=meta)``
+        for every layer; the same metadata serves all layers."""
+        n = len(seq_ids)
+        counts = [new_tokens] * n if isinstance(new_tokens, int) else list(new_tokens)
+        if len(counts) != n:
+            raise ValueError("one new-token count per sequence")
+        width = max(counts) if counts else 0
+        slots = []
+        for sid, c in zip(seq_ids, counts):
+            seq = self._seqs[sid]
+            row = [self._slot_for_append(seq) for _ in range(c)]
+            slots.extend(row + [-1] * (width - c))
+        lens = [self._seqs[s].length for s in seq_ids]
+        max_blocks = max((len(self._seqs[s].blocks) for s in seq_ids), default=1) or 1
+        table = [self._seqs[s].blocks + [0] * (max_blocks - len(self._seqs[s].blocks)) for s in seq_ids]
+        dev = self.device
+        cu = None
+        if any(c != width for c in counts):
+            # ragged chunks: rows are padded to `width`, the kernels get true bounds
+            raise NotImplementedError("per-sequence chunk lengths must be equal within one step")
+        return PagedAttentionMetadata(
+            block_tables=torch.tensor(table, dtype=torch.int32, device=dev).view(n, max_blocks),
+            context_lens=torch.tensor(lens, dtype=torch.int32, device=dev),
+            slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev),
+            max_context_len=max(lens, default=0),
+            cu_seqlens_q=cu)

@@ -1,0 +1,189 @@
+"""Attention layer: the reference's call signature, MI355X kernels underneath.
+
+Mirror of ``ironcore.layers.attention.Attention``
+(ironcore/layers/attention.py:24-253): same constructor argument, same
+attributes (attention.py:44-66), same ``forward(query, key, value,
+attention_mask=None)`` with ``query [b, sq, hn, hd]``, ``key``/``value``
+``[b, sk, gn, hd]`` and result ``[b, sq, hn*hd]`` (attention.py:208-253), same
+GQA head map (query head h reads KV head h // (hn // gn), attention.py:95-102)
+and the same scale 1/sqrt(d_model // hn) (attention.py:51,65,110).
+
+The block-KV-cache path is reached only through the two extra keyword
+arguments, so the reference's call site
+(ironcore/models/transformer.py:101-103) stays valid unchanged:
+
+    attn(query, key, value, attention_mask, kv_cache=layer_cache, attn_metadata=meta)
+
+appends the new ``key``/``value`` rows to the layer's block pool and attends
+against the cache (decode kernel for sq == 1, chunked-prefill kernel
+otherwise).  Without ``kv_cache`` the call is the reference's dense call; it
+runs on the same chunked-prefill kernel by viewing ``key``/``value`` as a pool
+with one block per sequence.  Every path runs the hand-written HIP kernels;
+there is no torch fallback.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+from torch import nn
+
+from .. import paged_ops
+from .module import BaseModule, get_model_dtype
+
+
+@dataclass
+class PagedAttentionMetadata:
+    """What one forward pass over a batch needs to know about the block KV
+    cache (built by ``ironcore_amd.kv_cache.PagedKVCache.prepare``).
+
+    block_tables   int32 [b, max_blocks]   pool block of each sequence block
+    context_lens   int32 [b]               tokens visible after this step's append
+    slot_mapping   int64 [b*sq]            pool slot of every new token, row-major
+                                           over (sequence, position); -1 = padding
+    max_context_len  host-side upper bound on context_lens
+    """
+    block_tables: torch.Tensor
+    context_lens: torch.Tensor
+    slot_mapping: torch.Tensor
+    max_context_len: int
+    cu_seqlens_q: Optional[torch.Tensor] = None   # int32 [b+1]; built on demand for prefill
+
+
+class Attention(BaseModule):
+    """Attention math only (no projections), as in the reference."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.num_attention_heads = config.model.num_attention_heads
+        self.tensor_model_parallel_size = config.trainer.tensor_model_parallel_size
+        self.head_dimension = config.model.d_model // self.num_attention_heads
+        self.num_local_attention_heads = self.num_attention_heads // self.tensor_model_parallel_size
+        self.num_local_attention_groups = (
+            config.model.num_attention_groups // self.tensor_model_parallel_size)
+        self.softmax = torch.nn.Softmax(dim=-1)
+        self.attn_dropout = nn.Dropout(config.model.dropout_attn)
+        self.scale_factor = self.head_dimension ** 0.5
+        self.mask_value = torch.finfo(get_model_dtype(config)).min
+
+    # ------------------------------------------------------------------ helpers
+    def _check_shapes(self, query, key, value):
+        if query.dim() != 4 or key.dim() != 4 or value.shape != key.shape:
+            raise ValueError("expected query [b, sq, hn, hd] and key/value [b, sk, gn, hd]")
+        b, sq, hn, hd = query.shape
+        if hn != self.num_local_attention_heads or key.shape[2] != self.num_local_attention_groups:
+            raise ValueError(
+                f"got {hn} query / {key.shape[2]} KV heads, layer has "
+                f"{self.num_local_attention_heads} / {self.num_local_attention_groups}")
+        if hd != self.head_dimension or key.shape[3] != hd:
+            raise ValueError(f"head dimension {hd} != d_model // heads = {self.head_dimension}")
+        if self.training and self.config.model.dropout_attn > 0.0:
+            raise NotImplementedError("attention dropout is a training feature; the paged "
+                                      "kernels implement the inference path (dropout_attn == 0 or eval())")
+
+    def _mask_is_causal(self, attention_mask, sq, sk) -> bool:
+        """True for the lower-triangular mask the reference model builds
+        (ironcore/language_model.py:109-114,159), shifted when sq < sk; None
+        means every key is visible.  Anything else is rejected: the kernels
+        implement those two patterns."""
+        if attention_mask is None:
+            return False
+        i = torch.arange(sq, device=attention_mask.device).unsqueeze(1)
+        j = torch.arange(sk, device=attention_mask.device).unsqueeze(0)
+        want = (j <= (sk - sq) + i)
+        got = attention_mask != 0
+        if got.shape[-2:] != (sq, sk):
+            raise ValueError(f"attention_mask must end in [{sq}, {sk}], got {tuple(attention_mask.shape)}")
+        if bool((got == want).all()):
+            return True
+        if bool(got.all()):
+            return False
+        raise NotImplementedError("only the causal mask (or no mask) is supported by the HIP attention path")
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, query, key, value, attention_mask=None, *, kv_cache=None, attn_metadata=None):
+        """query [b, sq, hn, hd]; key/value [b, sk, gn, hd]; returns [b, sq, hn*hd]."""
+        self._check_shapes(query, key, value)
+        if kv_cache is not None:
+            return self._paged(query, key, value, kv_cache, attn_metadata)
+        return self._dense(query, key, value, attention_mask)
+
+    def _dense(self, query, key, value, attention_mask):
+        b, sq, hn, hd = query.shape
+        sk, gn = key.shape[1], key.shape[2]
+        causal = self._mask_is_causal(attention_mask, sq, sk)
+        if query.dtype == torch.float32:
+            return self._dense_fp32(query, key, value, causal)
+        key, value = key.contiguous(), value.contiguous()
+        # one pool block per sequence: [b, gn, sk, hd] view of the [b, sk, gn, hd] rows
+        k_pool, v_pool = key.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)
+        dev = query.device
+        tables = torch.arange(b, dtype=torch.int32, device=dev).unsqueeze(1)
+        ctx = torch.full((b,), sk, dtype=torch.int32, device=dev)
+        cu = torch.arange(0, (b + 1) * sq, sq, dtype=torch.int32, device=dev)
+        out = paged_ops.paged_prefill(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx, cu, sq,
+                                      causal=causal, scale=1.0 / self.scale_factor)
+        return out.view(b, sq, hn * hd)
+
+    def _dense_fp32(self, query, key, value, causal):
+        """fp32 has no MFMA path: every query row runs as one decode-kernel
+        sequence over the keys it may see (fp32 loads, fp32 arithmetic)."""
+        b, sq, hn, hd = query.shape
+        sk, gn = key.shape[1], key.shape[2]
+        dev = query.device
+        # The decode kernel loads whole 16-token tiles: give every sequence a
+        # block padded to a multiple of 16 rows (rows past sk are never visible).
+        sk16 = (sk + 15) // 16 * 16
+        k_rows = key.new_zeros(b, sk16, gn, hd)
+        v_rows = value.new_zeros(b, sk16, gn, hd)
+        k_rows[:, :sk] = key
+        v_rows[:, :sk] = value
+        k_pool, v_pool = k_rows.permute(0, 2, 1, 3), v_rows.permute(0, 2, 1, 3)
+        return _fp32_rows_via_decode(query, k_pool, v_pool,
+                                     torch.arange(b, dtype=torch.int32, device=dev).unsqueeze(1),
+                                     torch.full((b,), sk, dtype=torch.int32, device=dev), sk, causal,
+                                     1.0 / self.scale_factor)
+
+    def _paged(self, query, key, value, kv_cache, meta):
+        if meta is None:
+            raise ValueError("kv_cache needs attn_metadata")
+        b, sq, hn, hd = query.shape
+        gn = key.shape[2]
+        if key.shape[1] != sq:
+            raise ValueError("with a KV cache, key/value carry only the new tokens (sk == sq)")
+        k_pool, v_pool = kv_cache
+        paged_ops.kv_append(key.reshape(b * sq, gn, hd), value.reshape(b * sq, gn, hd), k_pool, v_pool,
+                            meta.slot_mapping)
+        scale = 1.0 / self.scale_factor
+        if sq == 1:
+            out = paged_ops.paged_decode(query.view(b, hn, hd), k_pool, v_pool, meta.block_tables,
+                                         meta.context_lens, meta.max_context_len, scale=scale)
+            return out.view(b, 1, hn * hd)
+        if query.dtype == torch.float32:
+            return _fp32_rows_via_decode(query, k_pool, v_pool, meta.block_tables, meta.context_lens,
+                                         meta.max_context_len, True, scale)
+        cu = meta.cu_seqlens_q
+        if cu is None:
+            cu = torch.arange(0, (b + 1) * sq, sq, dtype=torch.int32, device=query.device)
+        out = paged_ops.paged_prefill(query.reshape(b * sq, hn, hd), k_pool, v_pool, meta.block_tables,
+                                      meta.context_lens, cu, sq, causal=True, scale=scale)
+        return out.view(b, sq, hn * hd)
+
+
+def _fp32_rows_via_decode(query, k_pool, v_pool, block_tables, context_lens, max_context_len, causal, scale):
+    """Chunk attention in fp32: query row r of sequence i becomes one
+    decode-kernel sequence with context_lens[i] - (sq - 1 - r) visible tokens
+    (all of them when not causal), sharing sequence i's block-table row."""
+    b, sq, hn, hd = query.shape
+    dev = query.device
+    rows = torch.arange(b, device=dev).repeat_interleave(sq)
+    tables = block_tables.index_select(0, rows)
+    if causal:
+        back = (sq - 1 - torch.arange(sq, device=dev, dtype=torch.int32)).repeat(b)
+        ctx = (context_lens.index_select(0, rows) - back).to(torch.int32)
+    else:
+        ctx = context_lens.index_select(0, rows).contiguous()
+    out = paged_ops.paged_decode(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx,
+                                 max_context_len, scale=scale)
+    return out.view(b, sq, hn * hd)

@@ -1,0 +1,95 @@
+"""The drop-in Attention layer on the GPU against the oracle (the reference's
+dense attention): dense calls with the reference's signature, and paged calls
+through the two extra keyword arguments."""
+import pytest
+import torch
+
+from ironcore_amd import config as ic_config
+from ironcore_amd.kv_cache import PagedKVCache
+from ironcore_amd.layers import Attention
+from oracle import paged as oracle_paged
+from oracle.dense_attention import causal_offset_mask, dense_attention
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(heads, groups, hd, precision):
+    return ic_config.MainConfig(model=ic_config.ModelConfig(
+        d_model=heads * hd, num_attention_heads=heads, num_attention_groups=groups, head_dim=hd,
+        dropout_attn=0.0, precision=precision), trainer=ic_config.TrainerConfig(use_flash_attn=False))
+
+
+def _qkv(b, sq, sk, hn, gn, hd, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(b, sq, hn, hd, generator=g).to(dtype), torch.randn(b, sk, gn, hd, generator=g).to(dtype),
+            torch.randn(b, sk, gn, hd, generator=g).to(dtype))
+
+
+def test_constructor_attributes_match_reference(gpu):
+    attn = Attention(_cfg(8, 4, 64, "bf16"))
+    assert attn.num_attention_heads == 8 and attn.head_dimension == 64
+    assert attn.num_local_attention_heads == 8 and attn.num_local_attention_groups == 4
+    assert isinstance(attn.softmax, torch.nn.Softmax) and isinstance(attn.attn_dropout, torch.nn.Dropout)
+    assert attn.scale_factor == 8.0 and attn.mask_value == torch.finfo(torch.bfloat16).min
+    assert len(list(attn.parameters())) == 0
+
+
+@pytest.mark.parametrize("dtype,precision,tol", [(torch.bfloat16, "bf16", 2e-2), (torch.float16, "fp16", 2e-2),
+                                                 (torch.float32, "fp32", 1e-4)])
+@pytest.mark.parametrize("hn,gn,hd", [(8, 8, 64), (8, 2, 128), (12, 12, 64)])
+@pytest.mark.parametrize("masked", [True, False])
+def test_dense_call_matches_reference_arithmetic(gpu, dtype, precision, tol, hn, gn, hd, masked):
+    b, s = 2, 70
+    q, k, v = _qkv(b, s, s, hn, gn, hd, dtype, seed=hn + hd)
+    mask = torch.tril(torch.ones(s, s)).view(1, 1, s, s).expand(b, -1, -1, -1) if masked else None
+    want = dense_attention(q, k, v, mask)
+    attn = Attention(_cfg(hn, gn, hd, precision)).to(gpu).eval()
+    got = attn(q.to(gpu), k.to(gpu), v.to(gpu), None if mask is None else mask.to(gpu))
+    torch.cuda.synchronize()
+    assert got.shape == (b, s, hn * hd) and torch.isfinite(got.float()).all()
+    assert (got.cpu().float() - want.float()).abs().max().item() <= tol
+
+
+def test_dense_call_with_shorter_query(gpu):
+    q, k, v = _qkv(2, 5, 40, 4, 4, 128, torch.bfloat16, seed=1)
+    mask = causal_offset_mask(5, 40)
+    want = dense_attention(q, k, v, mask)
+    attn = Attention(_cfg(4, 4, 128, "bf16")).to(gpu).eval()
+    got = attn(q.to(gpu), k.to(gpu), v.to(gpu), mask.to(gpu))
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2
+
+
+def test_unsupported_mask_is_rejected_loudly(gpu):
+    q, k, v = _qkv(1, 8, 8, 4, 4, 64, torch.bfloat16, seed=2)
+    mask = torch.ones(1, 1, 8, 8)
+    mask[..., 3] = 0
+    attn = Attention(_cfg(4, 4, 64, "bf16")).to(gpu).eval()
+    with pytest.raises(NotImplementedError):
+        attn(q.to(gpu), k.to(gpu), v.to(gpu), mask.to(gpu))
+
+
+@pytest.mark.parametrize("dtype,precision,tol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "fp32", 1e-4)])
+def test_paged_prefill_then_decode_through_the_layer(gpu, dtype, precision, tol):
+    hn, gn, hd, b = 8, 4, 64, 3
+    attn = Attention(_cfg(hn, gn, hd, precision)).to(gpu).eval()
+    cache = PagedKVCache(1, 32, 16, gn, hd, dtype, gpu)
+    ids = [cache.add_sequence() for _ in range(b)]
+    # oracle-side cache with the same block ids
+    kp = torch.zeros(32, gn, 16, hd, dtype=dtype)
+    vp = torch.zeros_like(kp)
+    total = 0
+    for step, sq in enumerate([37, 1, 1, 12, 1]):
+        q, k, v = _qkv(b, sq, sq, hn, gn, hd, dtype, seed=100 + step)
+        meta = cache.prepare(ids, sq)
+        got = attn(q.to(gpu), k.to(gpu), v.to(gpu), None, kv_cache=cache.layer(0), attn_metadata=meta)
+        torch.cuda.synchronize()
+        oracle_paged.kv_append(kp, vp, k.reshape(b * sq, gn, hd), v.reshape(b * sq, gn, hd), meta.slot_mapping.cpu())
+        total += sq
+        want = oracle_paged.paged_prefill(q.reshape(b * sq, hn, hd), kp, vp, meta.block_tables.cpu(),
+                                          meta.context_lens.cpu(),
+                                          torch.arange(0, (b + 1) * sq, sq, dtype=torch.int32)).view(b, sq, -1)
+        assert meta.context_lens.tolist() == [total] * b
+        assert (got.cpu().float() - want.float()).abs().max().item() <= tol, f"step {step}"
+    bits = torch.int16 if dtype != torch.float32 else torch.int32
+    assert torch.equal(cache.k_pools[0].cpu().view(bits), kp.view(bits))
+    assert torch.equal(cache.v_pools[0].cpu().view(bits), vp.view(bits))

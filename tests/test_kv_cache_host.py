@@ -1,0 +1,69 @@
+"""Host logic of the block KV cache: allocation, slot mapping, prefix sharing
+with copy-on-write.  CPU tensors (no kernel is called)."""
+import pytest
+import torch
+
+from ironcore_amd.kv_cache import BlockAllocator, OutOfBlocks, PagedKVCache
+
+
+def test_allocator_refcounts():
+    a = BlockAllocator(3)
+    b0, b1 = a.allocate(), a.allocate()
+    assert {b0, b1} == {0, 1} and a.num_free == 1
+    a.share(b0)
+    a.release(b0)
+    assert a.ref_count(b0) == 1 and a.num_free == 1
+    a.release(b0)
+    assert a.num_free == 2
+    with pytest.raises(ValueError):
+        a.release(b0)
+    a.allocate(), a.allocate()
+    with pytest.raises(OutOfBlocks):
+        a.allocate()
+
+
+def test_prepare_builds_tables_slots_and_lengths():
+    cache = PagedKVCache(2, 8, 16, 2, 8, torch.float32, "cpu")
+    s0, s1 = cache.add_sequence(), cache.add_sequence()
+    meta = cache.prepare([s0, s1], 20)
+    assert meta.context_lens.tolist() == [20, 20] and meta.max_context_len == 20
+    assert meta.block_tables.shape == (2, 2)
+    t = meta.block_tables.tolist()
+    assert len({*t[0], *t[1]}) == 4
+    want = [t[i][p // 16] * 16 + p % 16 for i in range(2) for p in range(20)]
+    assert meta.slot_mapping.tolist() == want
+    meta = cache.prepare([s0, s1], 1)
+    assert meta.context_lens.tolist() == [21, 21]
+    assert meta.slot_mapping.tolist() == [t[0][1] * 16 + 4, t[1][1] * 16 + 4]
+    cache.free_sequence(s0)
+    assert cache.allocator.num_free == 6
+
+
+def test_fork_aliases_full_blocks_and_copies_the_partial_one():
+    cache = PagedKVCache(1, 8, 16, 1, 4, torch.float32, "cpu")
+    s = cache.add_sequence()
+    cache.prepare([s], 40)                      # 2 full blocks + 8 tokens
+    blocks = cache.blocks(s)
+    cache.k_pools[0, blocks[2]].fill_(7.0)
+    c = cache.fork(s)
+    cb = cache.blocks(c)
+    assert cb[:2] == blocks[:2] and cb[2] != blocks[2]
+    assert cache.allocator.ref_count(blocks[0]) == 2
+    assert torch.equal(cache.k_pools[0, cb[2]], cache.k_pools[0, blocks[2]])
+    m = cache.prepare([s, c], 1)                # both append privately
+    assert m.slot_mapping.tolist() == [blocks[2] * 16 + 8, cb[2] * 16 + 8]
+    cache.free_sequence(s)
+    assert cache.allocator.ref_count(blocks[0]) == 1
+
+
+def test_append_into_shared_block_copies_on_write():
+    cache = PagedKVCache(1, 8, 16, 1, 4, torch.float32, "cpu")
+    s = cache.add_sequence()
+    cache.prepare([s], 32)                      # exactly 2 full blocks
+    c = cache.fork(s)                           # aliases both
+    # rewind the child by hand into the shared last block to force a write there
+    cache._seqs[c].length = 20
+    m = cache.prepare([c], 1)
+    new_blk = cache.blocks(c)[1]
+    assert new_blk != cache.blocks(s)[1]
+    assert m.slot_mapping.tolist() == [new_blk * 16 + 4]
