@@ -20,7 +20,7 @@ LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libironcore_paged.so"
 OBJ_DIR = PKG / "build" / "obj"
 
-SOURCES = ["ic_api.hip", "kv_append.hip", "paged_decode.hip", "paged_prefill.hip"]
+SOURCES = ["ic_api.hip", "kv_append.hip", "paged_decode.hip", "paged_decode_gqa.hip", "paged_prefill.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -42,9 +42,16 @@ def _hipcc() -> str:
     return exe
 
 
+# Per-file flags.  The prefill kernel keeps its MFMA accumulators in ordinary
+# VGPRs: the softmax rescales them with VALU instructions, and the AGPR form
+# costs a register copy each way per tile.
+PER_SOURCE_FLAGS = {"paged_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def _compile(src: str, extra: list[str]) -> Path:
     obj = OBJ_DIR / (src + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src, []), *extra, "-c", str(CSRC / src),
+           "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

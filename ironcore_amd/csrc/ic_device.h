@@ -41,6 +41,10 @@ struct Bf16 {
                                             __builtin_bit_cast(bf16x2_t, b.w[i]), acc, false);
     return acc;
   }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b),
+                                           acc, false);
+  }
   static __device__ __forceinline__ void widen(const Vec16 &a, float *f) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -60,6 +64,9 @@ struct F16 {
       acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a.w[i]),
                                    __builtin_bit_cast(f16x2_t, b.w[i]), acc, false);
     return acc;
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
   }
   static __device__ __forceinline__ void widen(const Vec16 &a, float *f) {
 #pragma unroll
@@ -103,6 +110,8 @@ constexpr int kDppQuadXor1 = 0xB1;      // quad_perm:[1,0,3,2]
 constexpr int kDppQuadXor2 = 0x4E;      // quad_perm:[2,3,0,1]
 constexpr int kDppRowHalfMirror = 0x141;  // lane i <- lane 7-i within each 8
 constexpr int kDppRowMirror = 0x140;      // lane i <- lane 15-i within each 16
+constexpr int kDppRowRor4 = 0x124;        // lane i <- lane (i+4)%16 within each 16
+constexpr int kDppRowRor8 = 0x128;        // lane i <- lane (i+8)%16 within each 16
 
 template <int LANES>
 __device__ __forceinline__ float group_sum(float x) {

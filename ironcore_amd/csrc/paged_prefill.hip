@@ -11,13 +11,16 @@
 // A dense contraction, so it runs on the matrix cores
 // (v_mfma_f32_32x32x16 bf16/f16, fp32 accumulate), flash-attention style:
 //
-//  * grid = (query tile of 128 rows, query head, sequence); 4 waves, each
-//    owning 32 query rows for the whole K/V sweep.  The wave's Q rows stay in
-//    registers as MFMA B operands.
+//  * grid = (query tile of 256 rows, query head, sequence); 4 waves, each
+//    owning two 32-row query blocks for the whole K/V sweep (128-row tiles
+//    with one block per wave for short chunks).  The wave's Q rows stay in
+//    registers as MFMA B operands; every K / V^T operand read from LDS feeds
+//    both blocks.
 //  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Each thread
-//    fetches its 16-byte pieces of the next tile through the block table
-//    while the current tile is being used, then parks them in LDS row-major
-//    ([token][dim], padded pitch).
+//    fetches its 16-byte pieces through the block table two tiles ahead
+//    (table entries are wave-uniform scalar loads), then parks them in
+//    double-buffered LDS, row-major ([token][dim], padded pitch).  One
+//    barrier per tile.
 //  * Scores are computed TRANSPOSED, S^T = K Q^T: in the MFMA result layout a
 //    lane then holds one query column, so the softmax row maximum and row sum
 //    are in-lane reductions plus one exchange between the two lane halves,
@@ -69,6 +72,7 @@ struct PrefillKP {
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
+constexpr float kLazySlack = 8.0f;  // log2 units
 
 // MFMA wrappers per element type: operands are 8 packed 16-bit values.
 struct MmaBf16 {
@@ -94,28 +98,39 @@ struct MmaF16 {
   }
 };
 
-constexpr int kPrefillThreads = 256;
-constexpr int kBM = 128;  // query rows per workgroup (32 per wave)
-constexpr int kBN = 64;   // tokens per K/V tile
+#ifndef IC_PREFILL_QB
+#define IC_PREFILL_QB 1
+#endif
 
-template <class M, int HD>
+constexpr int kPrefillThreads = 256;
+constexpr int kBN = 64;  // tokens per K/V tile
+
+// QB = 32-row query blocks per wave: a workgroup covers 4*32*QB query rows.
+// With QB = 2 every K / V^T operand read from LDS feeds two MFMAs, which
+// halves the LDS traffic per flop, and the softmax of one block overlaps the
+// matrix work of the other.
+// SINGLE: every sequence is one pool block (a dense [b, sk, gn, hd] tensor
+// viewed as a pool); otherwise blocks are a power of two >= 16 tokens long.
+template <class M, int HD, int QB, bool SINGLE>
 __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const PrefillKP p) {
   using T = typename M::T;
+  constexpr int BM = 4 * 32 * QB;      // query rows per workgroup
   constexpr int KS = HD / 16;          // k-steps of the QK contraction
   constexpr int OB = HD / 32;          // 32-wide blocks of the output head dim
   constexpr int TB = kBN / 32;         // 32-token blocks per tile
   constexpr int CPR = HD / 8;          // 16-byte chunks per token row
-  constexpr int NCH = kBN * CPR / kPrefillThreads;  // chunks per thread per tile
+  constexpr int RPP = kPrefillThreads / CPR;         // token rows staged per pass of the workgroup
+  constexpr int NCH = kBN / RPP;                     // passes (= chunks per thread) per tile
   constexpr int KP = HD * 2 + 16;      // K tile pitch in bytes (bank-conflict-free b128 reads)
   constexpr int VP = HD * 2 + 64;      // V tile pitch in bytes (conflict-free transposing reads)
-  static_assert(kBN * CPR % kPrefillThreads == 0, "tile staging shape");
+  static_assert(kBN % RPP == 0 && RPP % 16 == 0, "tile staging shape");
 
-  __shared__ __attribute__((aligned(16))) char s_k[kBN * KP];
-  __shared__ __attribute__((aligned(16))) char s_v[kBN * VP];
+  __shared__ __attribute__((aligned(16))) char s_k[2][kBN * KP];
+  __shared__ __attribute__((aligned(16))) char s_v[2][kBN * VP];
 
   const int seq = blockIdx.z;
   const int h = blockIdx.y;
-  const int q0 = blockIdx.x * kBM;
+  const int q0 = blockIdx.x * BM;
   const int q_lo = p.cu_seqlens_q[seq];
   int L = p.context_lens[seq];
   int C = p.cu_seqlens_q[seq + 1] - q_lo;
@@ -127,187 +142,251 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;
-  const int n = lane & 31;   // query column of this lane within the wave's 32 rows
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int n = lane & 31;   // query column of this lane within a 32-row block
   const int hh = lane >> 5;  // which half of each k-step this lane feeds
 
-  const int my_q = q0 + wave * 32 + n;
-  const bool q_valid = my_q < C;
-  const int64_t q_row = q_lo + (q_valid ? my_q : C - 1);
-  // last key this query row may see
-  const int limit = p.causal ? P + (q_valid ? my_q : C - 1) : L - 1;
-
-  Vec16 qf[KS];
+  // ---- query rows: registers for the whole sweep, as MFMA B operands ------------
+  int limit[QB];      // last key each query row may see
+  int my_q[QB];
+  Vec16 qf[QB][KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    qf[ks] = load16(p.q + (q_row * p.q_stride_token + (int64_t)h * HD + ks * 16 + hh * 8) * 2);
-
-  f32x16_t o[OB];
+  for (int qb = 0; qb < QB; ++qb) {
+    my_q[qb] = q0 + (wave * QB + qb) * 32 + n;
+    const int row = my_q[qb] < C ? my_q[qb] : C - 1;
+    limit[qb] = p.causal ? P + row : L - 1;
 #pragma unroll
-  for (int ob = 0; ob < OB; ++ob)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) o[ob][i] = 0.f;
-  float m = kNegInf, l = 0.f;
+    for (int ks = 0; ks < KS; ++ks)
+      qf[qb][ks] = load16(p.q + ((q_lo + row) * p.q_stride_token + (int64_t)h * HD + ks * 16 + hh * 8) * 2);
+  }
 
-  int kv_end = p.causal ? P + q0 + kBM : L;  // keys any row of this tile can see
+  f32x16_t o[QB][OB];
+  float m[QB], l[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m[qb] = kNegInf;
+    l[qb] = 0.f;
+#pragma unroll
+    for (int ob = 0; ob < OB; ++ob)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[qb][ob][i] = 0.f;
+  }
+
+  int kv_end = p.causal ? P + q0 + BM : L;  // keys any row of this workgroup can see
   kv_end = kv_end < L ? kv_end : L;
   const int n_tiles = (kv_end + kBN - 1) / kBN;
 
-  // ---- tile staging: global -> registers -> LDS --------------------------------
+  // ---- tile staging: global -> registers (one tile ahead) -> LDS -------------------
+  // In one pass the workgroup covers RPP consecutive token rows, a wave WR of
+  // them.  Pool blocks are a power of two >= 16 rows long (or the sequence is a
+  // single block), so the rows of one wave's pass lie inside one block: table
+  // entry, offset in the block and base address are wave-uniform scalar work
+  // and a thread only adds a fixed offset.
+  constexpr int WR = kWave / CPR;  // rows one wave stages per pass
+  static_assert(WR <= 16 && 16 % WR == 0, "a wave's pass must stay inside a 16-row group");
+  const int row0 = tid / CPR;
+  const int cc = tid - row0 * CPR;
+  const uint32_t thr_off = (uint32_t)(((row0 - wave * WR) * p.stride_token + cc * 8) * 2);
+  const int64_t head_off = (int64_t)kvh * p.stride_head;
   Vec16 kst[NCH], vst[NCH];
   auto fetch = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int chunk = tid + kPrefillThreads * i;
-      const int row = chunk / CPR;
-      const int cc = chunk - row * CPR;
-      const int tok = tile * kBN + row;
-      kst[i] = Vec16{{0u, 0u, 0u, 0u}};
-      vst[i] = Vec16{{0u, 0u, 0u, 0u}};
-      if (tok < L) {
-        int blk, off;
-        if (p.block_shift >= 0) {
-          blk = tok >> p.block_shift;
-          off = tok & (p.block_size - 1);
-        } else {
-          blk = tok / p.block_size;
-          off = tok - blk * p.block_size;
+      const int first = tile * kBN + i * RPP + wave * WR;  // this wave's first row of the pass
+      int blk = SINGLE ? 0 : first >> p.block_shift;
+      const int rem = SINGLE ? first : first & (p.block_size - 1);
+      blk = blk < p.bt_stride ? blk : (int)p.bt_stride - 1;
+      int64_t phys = __builtin_amdgcn_readfirstlane(p.block_tables[seq * p.bt_stride + blk]);
+      // A corrupt table entry must not become an out-of-pool address.
+      phys = phys < 0 ? 0 : phys;
+      phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
+      const int64_t base = (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2;
+      if (first + WR <= L) {
+        kst[i] = load16(p.k_pool + base + thr_off);
+        vst[i] = load16(p.v_pool + base + thr_off);
+      } else {  // the pass reaches past the context: those rows stay zero
+        kst[i] = Vec16{{0u, 0u, 0u, 0u}};
+        vst[i] = Vec16{{0u, 0u, 0u, 0u}};
+        if (tile * kBN + i * RPP + row0 < L) {
+          kst[i] = load16(p.k_pool + base + thr_off);
+          vst[i] = load16(p.v_pool + base + thr_off);
         }
-        blk = blk < p.bt_stride ? blk : (int)p.bt_stride - 1;
-        int64_t phys = p.block_tables[seq * p.bt_stride + blk];
-        // A corrupt table entry must not become an out-of-pool address.
-        phys = phys < 0 ? 0 : phys;
-        phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
-        const int64_t at =
-            (phys * p.stride_block + kvh * p.stride_head + off * p.stride_token + cc * 8) * 2;
-        kst[i] = load16(p.k_pool + at);
-        vst[i] = load16(p.v_pool + at);
       }
     }
   };
-  auto park = [&]() {
+  const int park_k = row0 * KP + cc * 16;
+  const int park_v = row0 * VP + cc * 16;
+  auto park = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int chunk = tid + kPrefillThreads * i;
-      const int row = chunk / CPR;
-      const int cc = chunk - row * CPR;
-      store16(s_k + row * KP + cc * 16, kst[i]);
-      store16(s_v + row * VP + cc * 16, vst[i]);
+      store16(s_k[buf] + park_k + i * RPP * KP, kst[i]);
+      store16(s_v[buf] + park_v + i * RPP * VP, vst[i]);
     }
   };
 
   // per-lane LDS offsets
-  const int k_lane = n * KP + hh * 16;                                   // + tb*32*KP + ks*32
+  const int k_lane = n * KP + hh * 16;  // + tb*32*KP + ks*32
   const int v_lane = (4 * hh + (lane & 15) / 4) * VP + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
-  fetch(0);
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    park();
-    __syncthreads();
-    if (tile + 1 < n_tiles) fetch(tile + 1);
+  auto compute = [&](int tile, int buf) {
+    const char *sk = s_k[buf];
+    const char *sv = s_v[buf];
+    // A 32-row block whose every row ends before this tile starts has nothing to do.
+    bool active[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+      active[qb] = !p.causal || tile * kBN <= P + q0 + (wave * QB + qb) * 32 + 31;
+    if (!active[QB - 1]) return;  // blocks are ordered: the last one sees the most keys
 
     // ---- S^T = K Q^T ------------------------------------------------------------
-    f32x16_t s[TB];
+    f32x16_t s[QB][TB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[qb][tb][i] = 0.f;
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[tb][i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const Vec16 a = load16(s_k + k_lane + tb * 32 * KP + ks * 32);
-        s[tb] = M::mma(a, qf[ks], s[tb]);
+        const Vec16 a = load16(sk + k_lane + tb * 32 * KP + ks * 32);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) s[qb][tb] = M::mma(a, qf[qb][ks], s[qb][tb]);
       }
     }
-    // s[tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n)
+    // s[qb][tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n of block qb)
     const int tok_base = tile * kBN + 4 * hh;
-    const bool need_mask = p.causal ? (tile * kBN + kBN - 1 > P + q0) : (tile * kBN + kBN > L);
-    float mx = kNegInf;
+    const bool need_mask = p.causal ? (tile * kBN + kBN - 1 > P + q0 + wave * QB * 32)
+                                    : (tile * kBN + kBN > L);
+    Vec16 pb[QB][kBN / 16];
+    if (need_mask) {  // tiles that touch the causal diagonal (or the context end)
 #pragma unroll
-    for (int tb = 0; tb < TB; ++tb) {
+      for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float x = s[tb][i] * p.scale_log2e;
-        if (need_mask) {
-          const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
-          x = tok > limit ? kNegInf : x;
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
+            s[qb][tb][i] = tok > limit[qb] ? kNegInf : s[qb][tb][i];
+          }
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      // Row maximum on the raw scores (the scale is positive), one exchange
+      // between the lane halves, then into log2 units.
+      float mx = kNegInf;
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[qb][tb][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * p.scale_log2e;
+      // Lazy reference maximum: it moves (and the accumulators are rescaled)
+      // only when some row's maximum rises by more than 2^kLazySlack above
+      // it.  Until then probabilities may exceed 1 (<= 2^kLazySlack), which
+      // fp32 sums and the 16-bit P operand hold without loss of accuracy.
+      if (__any(mx > m[qb] + kLazySlack)) {
+        const float m_new = fmaxf(m[qb], mx);
+        const float alpha = (m[qb] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[qb] - m_new);
+        m[qb] = m_new;
+        l[qb] *= alpha;
+#pragma unroll
+        for (int ob = 0; ob < OB; ++ob)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[qb][ob][i] *= alpha;
+      }
+      const float neg_ms = (m[qb] == kNegInf) ? 0.f : -m[qb];
+      float ps = 0.f;
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb) {
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][tb][i], p.scale_log2e, neg_ms));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][tb][i + 1], p.scale_log2e, neg_ms));
+          ps += p0 + p1;
+          pb[qb][2 * tb + i / 8].w[(i & 7) / 2] = M::pack2(p0, p1);
         }
-        s[tb][i] = x;
-        mx = fmaxf(mx, x);
       }
+      l[qb] += ps;
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m, mx);
-    const float ms = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m - ms);
-    m = m_new;
-    float ps = 0.f;
-    Vec16 pb[kBN / 16];
-#pragma unroll
-    for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(s[tb][i] - ms);
-        const float p1 = __builtin_amdgcn_exp2f(s[tb][i + 1] - ms);
-        ps += p0 + p1;
-        pb[2 * tb + i / 8].w[(i & 7) / 2] = M::pack2(p0, p1);
-      }
-    }
-    l = l * alpha + ps;
-#pragma unroll
-    for (int ob = 0; ob < OB; ++ob)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[ob][i] *= alpha;
 
     // ---- O^T += V^T P^T -----------------------------------------------------------
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob) {
 #pragma unroll
       for (int kk = 0; kk < kBN / 16; ++kk) {
-        const char *at = s_v + v_lane + kk * 16 * VP + ob * 64;
+        const char *at = sv + v_lane + kk * 16 * VP + ob * 64;
         const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) s16x4_t *)(at));
         const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) s16x4_t *)(at + 8 * VP));
         const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        o[ob] = M::mma(__builtin_bit_cast(Vec16, both), pb[kk], o[ob]);
+        const Vec16 a = __builtin_bit_cast(Vec16, both);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) o[qb][ob] = M::mma(a, pb[qb][kk], o[qb][ob]);
       }
     }
+  };
+
+  // Pipeline: LDS[t&1] holds tile t while the registers carry tile t+1.  One
+  // barrier per tile.
+  fetch(0);
+  park(0);
+  if (n_tiles > 1) fetch(1);
+  __syncthreads();
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    compute(tile, tile & 1);
+    if (tile + 1 < n_tiles) park((tile + 1) & 1);
     __syncthreads();
+    if (tile + 2 < n_tiles) fetch(tile + 2);
   }
 
   // ---- normalise and store -------------------------------------------------------
-  l += __shfl_xor(l, 32, kWave);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  if (q_valid) {
-    T *orow = reinterpret_cast<T *>(p.out) + (q_lo + my_q) * p.out_stride_token + (int64_t)h * HD;
 #pragma unroll
-    for (int ob = 0; ob < OB; ++ob) {
+  for (int qb = 0; qb < QB; ++qb) {
+    float lt = l[qb] + __shfl_xor(l[qb], 32, kWave);
+    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    if (my_q[qb] < C) {
+      T *orow = reinterpret_cast<T *>(p.out) + (q_lo + my_q[qb]) * p.out_stride_token + (int64_t)h * HD;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = ob * 32 + 4 * hh + 8 * j;
-        uint2 w;
-        w.x = M::pack2(o[ob][4 * j] * inv, o[ob][4 * j + 1] * inv);
-        w.y = M::pack2(o[ob][4 * j + 2] * inv, o[ob][4 * j + 3] * inv);
-        *reinterpret_cast<uint2 *>(orow + d) = w;
+      for (int ob = 0; ob < OB; ++ob) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int d = ob * 32 + 4 * hh + 8 * j;
+          uint2 w;
+          w.x = M::pack2(o[qb][ob][4 * j] * inv, o[qb][ob][4 * j + 1] * inv);
+          w.y = M::pack2(o[qb][ob][4 * j + 2] * inv, o[qb][ob][4 * j + 3] * inv);
+          *reinterpret_cast<uint2 *>(orow + d) = w;
+        }
       }
     }
   }
 }
 
-template <class M>
+template <class M, int QB, bool SINGLE>
 int launch_hd(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
-  const dim3 grid((a.max_chunk_len + kBM - 1) / kBM, a.hn, a.n_seqs);
+  constexpr int BM = 4 * 32 * QB;
+  const dim3 grid((a.max_chunk_len + BM - 1) / BM, a.hn, a.n_seqs);
   switch (a.hd) {
     case 64:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 64>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 64, QB, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     case 128:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 128>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 128, QB, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     default:
       return IC_ERR_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;
+}
+
+template <class M>
+int launch_mode(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
+  constexpr int QB = IC_PREFILL_QB;
+  // A one-column block table means one block per sequence, of any length.
+  if (a.block_table_stride == 1) return launch_hd<M, QB, true>(kp, a, stream);
+  if (kp.block_shift < 4) return IC_ERR_UNSUPPORTED;  // power-of-two blocks of >= 16 tokens
+  return launch_hd<M, QB, false>(kp, a, stream);
 }
 
 }  // namespace
@@ -335,11 +414,11 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   kp.group = a.hn / a.gn;
   kp.causal = a.causal;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
-  if ((int64_t)a.max_chunk_len + kBM - 1 >= (int64_t)65535 * kBM || a.hn > 65535 || a.n_seqs > 65535)
+  if ((int64_t)a.max_chunk_len >= (int64_t)65535 * 128 || a.hn > 65535 || a.n_seqs > 65535)
     return IC_ERR_UNSUPPORTED;
   switch (a.dtype) {
-    case IC_DTYPE_BF16: return launch_hd<MmaBf16>(kp, a, stream);
-    case IC_DTYPE_F16: return launch_hd<MmaF16>(kp, a, stream);
+    case IC_DTYPE_BF16: return launch_mode<MmaBf16>(kp, a, stream);
+    case IC_DTYPE_F16: return launch_mode<MmaF16>(kp, a, stream);
     default: return IC_ERR_UNSUPPORTED;  // fp32 has no MFMA path here
   }
 }
