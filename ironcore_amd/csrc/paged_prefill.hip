@@ -11,16 +11,16 @@
 // A dense contraction, so it runs on the matrix cores
 // (v_mfma_f32_32x32x16 bf16/f16, fp32 accumulate), flash-attention style:
 //
-//  * grid = (query tile of 256 rows, query head, sequence); 4 waves, each
-//    owning two 32-row query blocks for the whole K/V sweep (128-row tiles
-//    with one block per wave for short chunks).  The wave's Q rows stay in
-//    registers as MFMA B operands; every K / V^T operand read from LDS feeds
-//    both blocks.
+//  * One workgroup = a query tile of 128 rows of one query head; 4 waves, each
+//    owning a 32-row query block for the whole K/V sweep, two workgroups per
+//    CU.  The wave's Q rows stay in registers as MFMA B operands.  Workgroup
+//    ids are laid out so that all tiles and heads that read the same K/V rows
+//    run on one XCD and share its L2.
 //  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Each thread
-//    fetches its 16-byte pieces through the block table two tiles ahead
-//    (table entries are wave-uniform scalar loads), then parks them in
-//    double-buffered LDS, row-major ([token][dim], padded pitch).  One
-//    barrier per tile.
+//    fetches its 16-byte pieces through the block table one tile ahead
+//    (table entry and base address are wave-uniform scalar work), then parks
+//    them in double-buffered LDS, row-major ([token][dim], padded pitch).
+//    One barrier per tile.
 //  * Scores are computed TRANSPOSED, S^T = K Q^T: in the MFMA result layout a
 //    lane then holds one query column, so the softmax row maximum and row sum
 //    are in-lane reductions plus one exchange between the two lane halves,
@@ -67,6 +67,9 @@ struct PrefillKP {
   int block_size;
   int block_shift;  // log2(block_size) when it is a power of two, else -1
   int group;        // query heads per KV head
+  int gn;           // KV heads
+  int n_units;      // n_seqs * gn
+  int n_qtiles;     // query tiles per chunk (grid sizing)
   int causal;
   float scale_log2e;
 };
@@ -103,6 +106,7 @@ struct MmaF16 {
 #endif
 
 constexpr int kPrefillThreads = 256;
+constexpr int kXcds = 8;
 constexpr int kBN = 64;  // tokens per K/V tile
 
 // QB = 32-row query blocks per wave: a workgroup covers 4*32*QB query rows.
@@ -128,9 +132,21 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   __shared__ __attribute__((aligned(16))) char s_k[2][kBN * KP];
   __shared__ __attribute__((aligned(16))) char s_v[2][kBN * VP];
 
-  const int seq = blockIdx.z;
-  const int h = blockIdx.y;
-  const int q0 = blockIdx.x * BM;
+  // XCD-aware placement.  Workgroups are dealt to the 8 XCDs round-robin by
+  // their linear id, and each XCD has its own L2.  All workgroups that read
+  // the same K/V rows (one (sequence, KV head) unit: its G query heads x its
+  // query tiles) get ids that differ by a multiple of 8, so they share an L2
+  // and the rows come from HBM once.
+  const int per_unit = p.group * p.n_qtiles;
+  const int slice = blockIdx.x / (kXcds * per_unit);
+  const int within = blockIdx.x - slice * (kXcds * per_unit);
+  const int unit = slice * kXcds + (within % kXcds);  // (sequence, KV head)
+  if (unit >= p.n_units) return;
+  const int r = within / kXcds;
+  const int seq = unit / p.gn;
+  const int kvh = unit - seq * p.gn;
+  const int h = kvh * p.group + r / p.n_qtiles;
+  const int q0 = (r % p.n_qtiles) * BM;
   const int q_lo = p.cu_seqlens_q[seq];
   int L = p.context_lens[seq];
   int C = p.cu_seqlens_q[seq + 1] - q_lo;
@@ -138,8 +154,6 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   if (C > L) C = L;  // a chunk cannot be longer than its context
   if (q0 >= C) return;
   const int P = L - C;  // cached prefix
-  const int kvh = h / p.group;
-
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -364,9 +378,13 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
 }
 
 template <class M, int QB, bool SINGLE>
-int launch_hd(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
+int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
   constexpr int BM = 4 * 32 * QB;
-  const dim3 grid((a.max_chunk_len + BM - 1) / BM, a.hn, a.n_seqs);
+  kp.n_qtiles = (a.max_chunk_len + BM - 1) / BM;
+  const int64_t slices = (kp.n_units + kXcds - 1) / kXcds;
+  const int64_t wgs = slices * kXcds * kp.group * kp.n_qtiles;
+  if (wgs > 0x7fffffff) return IC_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs);
   switch (a.hd) {
     case 64:
       hipLaunchKernelGGL((paged_prefill_kernel<M, 64, QB, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
@@ -412,6 +430,9 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   for (int s = 0; s < 31; ++s)
     if ((1 << s) == a.pool.block_size) kp.block_shift = s;
   kp.group = a.hn / a.gn;
+  kp.gn = a.gn;
+  kp.n_units = a.n_seqs * a.gn;
+  kp.n_qtiles = 0;
   kp.causal = a.causal;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
   if ((int64_t)a.max_chunk_len >= (int64_t)65535 * 128 || a.hn > 65535 || a.n_seqs > 65535)
