@@ -280,47 +280,51 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   }
 }
 
-// Combine the split-K partials of one (sequence, query head).
-// grid = (hn, n_seqs), HD threads.  A pair's tiles are a contiguous run of the
-// batch-wide sequence, so the waves that touched it are
+constexpr int kReduceThreads = 256;
+
+// Combine the split-K partials of one pair (a KV head's query heads of one
+// sequence).  grid = (pairs per sequence, n_seqs).  A pair's tiles are a
+// contiguous run of the batch-wide sequence, so the waves that touched it are
 // first_tile / chunk .. last_tile / chunk and their partial ids follow.
 // Traffic is (hd+2)*4 bytes per partial, three orders of magnitude below the
 // K/V stream.
 template <class E, int HD, int GT>
-__global__ __launch_bounds__(HD) void paged_decode_reduce_kernel(const DecodeKP p) {
+__global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(const DecodeKP p) {
   using T = typename E::type;
-  const int h = blockIdx.x;
+  const int pair_in_seq = blockIdx.x;
   const int seq = blockIdx.y;
-  const int d = threadIdx.x;
-  T *o = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)h * HD + d;
+  const int kvh = pair_in_seq / p.nsub;
+  const int sub = pair_in_seq - kvh * p.nsub;
+  const int head0 = kvh * p.group + sub * GT;
+  const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+  T *orow = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)head0 * HD;
   const int cum = p.cum_blocks[seq];
   const int nb = p.cum_blocks[seq + 1] - cum;
-  if (nb == 0) {
-    *o = E::narrow(0.f);
+  if (nb == 0) {  // no visible token: zero rows
+    for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) orow[o] = E::narrow(0.f);
     return;
   }
-  const int kvh = h / p.group;
-  const int gi = h - kvh * p.group;
-  const int sub = gi / GT;
-  const int g = gi - sub * GT;
-  const int pair_in_seq = kvh * p.nsub + sub;
   const int64_t n_tiles = (int64_t)p.cum_blocks[p.n_seqs] * p.pairs_per_seq;
   const int64_t chunk = chunk_tiles(p, n_tiles);
   const int64_t first = (int64_t)cum * p.pairs_per_seq + (int64_t)pair_in_seq * nb;
   const int64_t w0 = first / chunk;
   const int64_t w1 = (first + nb - 1) / chunk;
-  if (w0 == w1) return;  // one wave covered the whole pair and wrote the row
+  if (w0 == w1) return;  // one wave covered the whole pair and wrote the rows
   const int64_t base = (int64_t)seq * p.pairs_per_seq + pair_in_seq;
-  float mx = kNegInf;
-  for (int64_t w = w0; w <= w1; ++w) mx = fmaxf(mx, p.part_ml[((w + base) * GT + g) * 2]);
-  float lsum = 0.f, a = 0.f;
-  for (int64_t w = w0; w <= w1; ++w) {
-    const int64_t slot = (w + base) * GT + g;
-    const float wt = __builtin_amdgcn_exp2f(p.part_ml[slot * 2] - mx);
-    lsum = __builtin_fmaf(p.part_ml[slot * 2 + 1], wt, lsum);
-    a = __builtin_fmaf(p.part_acc[slot * HD + d], wt, a);
+  for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) {
+    const int g = o / HD;
+    const int d = o - g * HD;
+    float mx = kNegInf;
+    for (int64_t w = w0; w <= w1; ++w) mx = fmaxf(mx, p.part_ml[((w + base) * GT + g) * 2]);
+    float lsum = 0.f, a = 0.f;
+    for (int64_t w = w0; w <= w1; ++w) {
+      const int64_t slot = (w + base) * GT + g;
+      const float wt = __builtin_amdgcn_exp2f(p.part_ml[slot * 2] - mx);
+      lsum = __builtin_fmaf(p.part_ml[slot * 2 + 1], wt, lsum);
+      a = __builtin_fmaf(p.part_acc[slot * HD + d], wt, a);
+    }
+    orow[o] = E::narrow(a / lsum);
   }
-  *o = E::narrow(a / lsum);
 }
 
 // Waves of the main kernel that one GPU holds at once, per kernel variant.
@@ -347,8 +351,8 @@ int launch_typed(DecodeKP &kp, int dtype, hipStream_t stream) {
     kp.n_waves = wgs * NW;
     hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
   }
-  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD, GT>), dim3(kp.hn, kp.n_seqs), dim3(HD), 0,
-                     stream, kp);
+  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD, GT>), dim3(kp.pairs_per_seq, kp.n_seqs),
+                     dim3(kReduceThreads), 0, stream, kp);
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;
 }
 
