@@ -45,7 +45,8 @@ def _hipcc() -> str:
 # Per-file flags.  The prefill kernel keeps its MFMA accumulators in ordinary
 # VGPRs: the softmax rescales them with VALU instructions, and the AGPR form
 # costs a register copy each way per tile.
-PER_SOURCE_FLAGS = {"paged_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+_VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+PER_SOURCE_FLAGS = {"paged_prefill.hip": _VGPR_FORM, "paged_decode_gqa.hip": _VGPR_FORM}
 
 
 def _compile(src: str, extra: list[str]) -> Path:

@@ -30,6 +30,7 @@ struct DecodeKP {
   int hn;
   int group;        // query heads per KV head
   int nsub;         // query sub-groups per KV head (ceil(group / GT))
+  int gt;           // query heads per sub-group (the stride of the partial arrays)
   int pairs_per_seq;  // gn * nsub
   int max_ctx;
   int n_waves;      // waves in the main kernel's grid

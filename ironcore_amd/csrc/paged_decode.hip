@@ -361,6 +361,7 @@ int launch_group(DecodeKP &kp, int gn, int dtype, hipStream_t stream) {
   const int G = kp.group;
   const int gt = decode_heads_per_wave(G);
   kp.nsub = (G + gt - 1) / gt;
+  kp.gt = gt;
   kp.pairs_per_seq = gn * kp.nsub;
   switch (gt) {
     case 1: return launch_typed<E, HD, 1>(kp, dtype, stream);
@@ -410,6 +411,7 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.hn = a.hn;
   kp.group = a.hn / a.gn;
   kp.nsub = 1;
+  kp.gt = 1;
   kp.pairs_per_seq = a.gn;
   kp.max_ctx = a.max_context_len;
   kp.n_waves = 0;

@@ -1,27 +1,36 @@
-// Paged decode for grouped-query attention (several query heads per KV head).
+// Paged decode for grouped-query attention (several query heads per KV head),
+// 16-bit element types, on the matrix cores.
 //
 // Same result, same balanced split-K bookkeeping, same partial format and
-// reduce pass as paged_decode.hip; what changes is how a tile's arithmetic is
-// laid over the lanes, because with G query heads per K/V byte the
-// single-head mapping runs out of VALU issue slots long before it runs out
-// of HBM bandwidth.  Per 16-token tile and G heads:
+// reduce pass as paged_decode.hip.  What changes is the arithmetic of a tile:
+// with G query heads per K/V byte the vector ALU runs out of issue slots long
+// before HBM runs out of bandwidth, so both products of a 16-token tile go to
+// MFMA with the (up to 16) query heads of the pair as one matrix dimension.
+// Nothing moves between lanes and nothing goes through LDS on the per-tile
+// path:
 //
-//  * q.k: ONE TOKEN PER QUAD.  Lane l holds a quarter (hd/4 dims) of token
-//    l/4's K row; the G query rows sit in LDS and are read as broadcasts.
-//    A score needs 2 DPP adds (quad_perm) instead of a 16-lane butterfly, and
-//    each lane ends with the G scores of ONE token, so the tile costs G
-//    v_exp per lane instead of 4 G.
-//  * Running maximum: kept per head as a wave-uniform reference and only
-//    moved when some score exceeds it by more than 2^5; until then no
-//    cross-lane reduction and no rescale of the accumulators happens at all
-//    (for iid scores that is the first tile of a segment and almost never
-//    again).  Probabilities stay <= 32 and the sum is exact in fp32.
-//  * p.v: probabilities go through a 256-byte LDS slab as packed 16-bit pairs
-//    (the reference rounds them to the element type too), V stays in the
-//    coalesced row mapping (16 bytes per lane), pairs of tokens are packed
-//    with v_perm_b32 and each head costs hd/8 v_dot2 per lane per 4 tokens.
+//  * S = K . Q^T   (v_mfma_f32_16x16x32, hd/32 of them).  A = the K tile
+//    straight from the 16-byte global loads: lane l supplies row l%16 and the
+//    8 dims 32j + 8(l/16) .. +7.  B = the query rows, held in registers for
+//    the whole segment: lane l supplies head l%16 (zero beyond the pair's
+//    heads), same dims.  The result leaves lane l with the scores of head
+//    l%16 for the four S rows 4(l/16) .. +3.
+//  * S row i is token (i/4) + 4(i%4) of the tile (a lane just loads that
+//    token's K row), so lane l owns tokens kg, kg+4, kg+8, kg+12 (kg = l/16):
+//    exactly the four k-elements lane l must supply for matrix A of the next
+//    product.  exp2 and the 16-bit rounding (the reference rounds the
+//    probabilities to the element type too) happen in place.
+//  * O += P . V    (v_mfma_f32_16x16x16, one per dim owned by a lane).  B = V:
+//    lane l loads dims (l%16)*hd/16 .. of tokens kg + 4i (coalesced rows) and
+//    packs token pairs with v_perm_b32; MFMA e covers dim (l%16)*hd/16 + e.
+//    The accumulators leave lane l with heads 4kg .. 4kg+3 of those dims.
+//  * Running maximum: a per-head reference that only moves when some score
+//    exceeds it by more than 2^5 (wave-uniform test); until then there is no
+//    cross-lane reduction and no rescale.  Row sums stay per lane and are
+//    folded once per segment.
 //
-// About 45 VALU issue slots per head per tile instead of 110.
+// Per tile and wave: hd/32 + hd/16 MFMAs and about 50 vector instructions,
+// whatever G is.
 #include "decode_common.h"
 #include "../../include/ironcore_paged.h"
 
@@ -32,53 +41,77 @@ namespace {
 
 constexpr float kLazyMaxSlack = 5.0f;  // log2 units
 
-__device__ __forceinline__ float dpp_max(float x, float y) { return fmaxf(x, y); }
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
-// max / sum over the 16 token slots of a tile: lanes l/4 (quads hold copies).
-__device__ __forceinline__ float token_max(float x) {
-  x = fmaxf(x, dpp_f32<kDppRowRor4>(x));
-  x = fmaxf(x, dpp_f32<kDppRowRor8>(x));
-  x = fmaxf(x, __shfl_xor(x, 16, kWave));
-  x = fmaxf(x, __shfl_xor(x, 32, kWave));
-  return x;
+struct Pair32 {
+  uint32_t lo, hi;
+};
+
+struct MfmaBf16 : Bf16 {
+  static __device__ __forceinline__ f32x4_t qk(const Vec16 &a, const Vec16 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4_t pv(const Pair32 &a, const Pair32 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
+                                                     __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const bf16x2_t v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+};
+
+struct MfmaF16 : F16 {
+  static __device__ __forceinline__ f32x4_t qk(const Vec16 &a, const Vec16 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4_t pv(const Pair32 &a, const Pair32 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                 __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    const f16x2_t v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+};
+
+// VW dwords (2*VW elements) of one V row.
+template <int VW>
+struct VChunk {
+  uint32_t w[VW];
+};
+template <int VW>
+__device__ __forceinline__ VChunk<VW> load_v(const void *p);
+template <>
+__device__ __forceinline__ VChunk<4> load_v<4>(const void *p) {
+  const Vec16 v = load16(p);
+  return VChunk<4>{{v.w[0], v.w[1], v.w[2], v.w[3]}};
 }
-__device__ __forceinline__ float token_sum(float x) {
-  x += dpp_f32<kDppRowRor4>(x);
-  x += dpp_f32<kDppRowRor8>(x);
-  x += __shfl_xor(x, 16, kWave);
-  x += __shfl_xor(x, 32, kWave);
-  return x;
+template <>
+__device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
+  const uint2 v = *reinterpret_cast<const uint2 *>(p);
+  return VChunk<2>{{v.x, v.y}};
 }
 
-#ifdef IC_GQA_WAVES_PER_EU
-#define IC_GQA_OCC __attribute__((amdgpu_waves_per_eu(IC_GQA_WAVES_PER_EU)))
-#else
-#define IC_GQA_OCC
-#endif
-
-template <class E, int HD, int GT, int BS, int NW>
-__global__ __launch_bounds__(NW *kWave) IC_GQA_OCC void paged_decode_gqa_kernel(const DecodeKP p) {
+template <class E, int HD, int BS, int NW>
+__global__ __launch_bounds__(NW *kWave) void paged_decode_gqa_kernel(const DecodeKP p) {
   using T = typename E::type;
-  static_assert(sizeof(T) == 2, "16-bit element types only");
   constexpr int ES = 2;
-  constexpr int DPL = HD / 4;       // K side: dims per lane (a quad covers one token row)
-  constexpr int NK = DPL / 8;       // K side: 16-byte loads per lane per tile
-  constexpr int LPR = HD / 8;       // V side: lanes sharing one token row
-  constexpr int RPL = kWave / LPR;  // V side: token rows per load instruction
-  constexpr int NLD = BS / RPL;     // V side: loads per tile = tokens per lane
+  constexpr int NK = HD / 32;  // q.k MFMAs = 16-byte K loads per lane per tile
+  constexpr int VE = HD / 16;  // V dims per lane = p.v MFMAs per tile
+  constexpr int VW = VE / 2;   // dwords per V load
+  constexpr int NT = 4;        // tokens per lane on the V side
   constexpr int SW = 4;
-  constexpr int NQ = (GT * HD / 8 + kWave - 1) / kWave;  // 16-byte q chunks per lane
-  static_assert(BS == 16 && (NLD == 2 || NLD == 4), "tile shape");
-
-  __shared__ __attribute__((aligned(16))) T s_q[NW][GT * HD];
-  __shared__ __attribute__((aligned(8))) T s_p[NW][RPL][GT][NLD];
+  static_assert(sizeof(T) == 2 && BS == 16 && (VW == 2 || VW == 4), "tile shape");
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int tq = lane >> 2;         // K side: token of this lane's quad
-  const int qc = lane & 3;          // K side: which quarter of the row
-  const int col = lane % LPR;       // V side
-  const int rowg = lane / LPR;      // V side
+  const int n = lane & 15;   // matrix column: head (q.k) or dim group (p.v)
+  const int kg = lane >> 4;  // this lane's tokens are kg, kg+4, kg+8, kg+12
 
   const int64_t wid = (int64_t)blockIdx.x * NW + wave;
   int64_t left;
@@ -88,202 +121,154 @@ __global__ __launch_bounds__(NW *kWave) IC_GQA_OCC void paged_decode_gqa_kernel(
   TileCursor peek = c;
   next_pair<BS>(p, peek);
   int seg_blk0 = c.blk;
+  const int GT = p.gt;
 
-  uint32_t k_off[NK], v_off[NLD];
+  // K side: S row n is token (n/4) + 4(n%4).
+  const int tok_k = (n >> 2) + 4 * (n & 3);
+  uint32_t k_off[NK], v_off[NT];
 #pragma unroll
-  for (int j = 0; j < NK; ++j) k_off[j] = (uint32_t)((tq * p.stride_token + qc * DPL + j * 8) * ES);
+  for (int j = 0; j < NK; ++j) k_off[j] = (uint32_t)((tok_k * p.stride_token + 32 * j + 8 * kg) * ES);
 #pragma unroll
-  for (int i = 0; i < NLD; ++i) v_off[i] = (uint32_t)(((i * RPL + rowg) * p.stride_token + col * 8) * ES);
+  for (int i = 0; i < NT; ++i) v_off[i] = (uint32_t)(((kg + 4 * i) * p.stride_token + n * VE) * ES);
 
-  // query rows of a pair: global -> registers (a segment ahead) -> LDS
-  auto fetch_q = [&](const TileCursor &tc, Vec16 *qq) {
+  auto pair_heads = [&](const TileCursor &tc, int &head0, int &heads) {
     const int kvh = tc.pair / p.nsub;
     const int sub = tc.pair - kvh * p.nsub;
-    const int head0 = kvh * p.group + sub * GT;
-    const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+    head0 = kvh * p.group + sub * GT;
+    heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+  };
+  // matrix B of q.k: head n, dims 32j + 8kg .. +7
+  auto fetch_q = [&](const TileCursor &tc, Vec16 *qq) {
+    int head0, heads;
+    pair_heads(tc, head0, heads);
 #pragma unroll
-    for (int u = 0; u < NQ; ++u) {
-      const int chunk = u * kWave + lane;  // 16-byte chunk of the [GT][HD] block
-      qq[u] = Vec16{{0u, 0u, 0u, 0u}};
-      if (chunk * 8 < heads * HD && tc.seq < p.n_seqs)
-        qq[u] = load16(p.q + (tc.seq * p.q_stride_seq + (int64_t)head0 * HD + chunk * 8) * ES);
+    for (int j = 0; j < NK; ++j) {
+      qq[j] = Vec16{{0u, 0u, 0u, 0u}};
+      if (n < heads && tc.seq < p.n_seqs)
+        qq[j] = load16(p.q + (tc.seq * p.q_stride_seq + (int64_t)(head0 + n) * HD + 32 * j + 8 * kg) * ES);
     }
   };
-  auto park_q = [&](const Vec16 *qq) {
-#pragma unroll
-    for (int u = 0; u < NQ; ++u) {
-      const int chunk = u * kWave + lane;
-      if (chunk * 8 < GT * HD) store16(&s_q[wave][chunk * 8], qq[u]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  };
-  Vec16 qnext[NQ];
-  fetch_q(c, qnext);
-  park_q(qnext);
+  Vec16 qreg[NK], qnext[NK];
+  fetch_q(c, qreg);
   fetch_q(peek, qnext);
 
-  float m[GT], l[GT], acc[GT][8];
+  float m = kNegInf;  // reference maximum of head n (the same in all four kg groups)
+  float l = 0.f;      // sum of this lane's probabilities of head n
+  f32x4_t acc[VE];    // acc[e][r]: head 4kg + r, dim n*VE + e
 #pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    m[g] = kNegInf;
-    l[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-  }
+  for (int e = 0; e < VE; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   auto finish_segment = [&]() {
-    const int kvh = c.pair / p.nsub;
-    const int sub = c.pair - kvh * p.nsub;
-    const int head0 = kvh * p.group + sub * GT;
-    const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+    int head0, heads;
+    pair_heads(c, head0, heads);
     const bool whole_pair = (seg_blk0 == 0 && c.blk == c.nb);
     const int64_t partial = wid + (int64_t)c.seq * p.pairs_per_seq + c.pair;
+    float lsum = l;
+    lsum += __shfl_xor(lsum, 16, kWave);
+    lsum += __shfl_xor(lsum, 32, kWave);
+    float lr[4];
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      if (g >= heads) break;
-      const float lsum = token_sum(l[g]);
-      // All V-side rows share the reference maximum: their accumulators just add.
-      float a[8];
+    for (int r = 0; r < 4; ++r) lr[r] = __shfl(lsum, 4 * kg + r, kWave);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        a[e] = acc[g][e];
-#pragma unroll
-        for (int step = LPR; step < kWave; step <<= 1) a[e] += __shfl_xor(a[e], step, kWave);
-      }
-      const int h = head0 + g;
-      if (rowg == 0) {  // one row writes dims col*8 .. col*8+7
+    for (int r = 0; r < 4; ++r) {
+      const int g = 4 * kg + r;
+      if (g < heads) {
         if (whole_pair) {
-          const float inv = 1.f / lsum;
-          T *o = reinterpret_cast<T *>(p.out) + c.seq * p.out_stride_seq + (int64_t)h * HD + col * 8;
+          const float inv = 1.f / lr[r];
+          uint32_t packed[VW];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = E::narrow(a[e] * inv);
+          for (int k = 0; k < VW; ++k) packed[k] = E::pack(acc[2 * k][r] * inv, acc[2 * k + 1][r] * inv);
+          char *o = p.out + (c.seq * p.out_stride_seq + (int64_t)(head0 + g) * HD + n * VE) * ES;
+          if (VW == 4)
+            store16(o, Vec16{{packed[0], packed[1], packed[2 % VW], packed[3 % VW]}});
+          else
+            *reinterpret_cast<uint2 *>(o) = make_uint2(packed[0], packed[1]);
         } else {
-          float *o = p.part_acc + (partial * GT + g) * HD + col * 8;
-          *reinterpret_cast<float4 *>(o) = make_float4(a[0], a[1], a[2], a[3]);
-          *reinterpret_cast<float4 *>(o + 4) = make_float4(a[4], a[5], a[6], a[7]);
+          float *o = p.part_acc + (partial * GT + g) * HD + n * VE;
+#pragma unroll
+          for (int k = 0; k < VE / 4; ++k)
+            *reinterpret_cast<float4 *>(o + 4 * k) =
+                make_float4(acc[4 * k][r], acc[4 * k + 1][r], acc[4 * k + 2][r], acc[4 * k + 3][r]);
         }
       }
-      if (!whole_pair && lane == 0) {
-        p.part_ml[(partial * GT + g) * 2] = m[g];
-        p.part_ml[(partial * GT + g) * 2 + 1] = lsum;
-      }
     }
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      m[g] = kNegInf;
-      l[g] = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    if (!whole_pair && kg == 0 && n < heads) {
+      p.part_ml[(partial * GT + n) * 2] = m;
+      p.part_ml[(partial * GT + n) * 2 + 1] = lsum;
     }
+    m = kNegInf;
+    l = 0.f;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (left > 0) {
       c = peek;
       seg_blk0 = 0;
-      park_q(qnext);
+#pragma unroll
+      for (int j = 0; j < NK; ++j) qreg[j] = qnext[j];
       next_pair<BS>(p, peek);
       fetch_q(peek, qnext);
     }
   };
 
-  auto consume = [&](Vec16 *kk, Vec16 *vv) {
-    // ---- scores: this lane's quad owns token tq of the tile ----------------------
-    float s[GT];
+  auto consume = [&](Vec16 *kk, VChunk<VW> *vv) {
+    // ---- scores of head n for tokens kg + 4r ------------------------------------
+    f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      float d = 0.f;
+    for (int j = 0; j < NK; ++j) s4 = E::qk(kk[j], qreg[j], s4);
+    float s[4];
 #pragma unroll
-      for (int j = 0; j < NK; ++j) d = E::dot(kk[j], load16(&s_q[wave][g * HD + qc * DPL + j * 8]), d);
-      d += dpp_f32<kDppQuadXor1>(d);
-      d += dpp_f32<kDppQuadXor2>(d);
-      s[g] = d * p.scale_log2e;
-    }
-    if (c.blk == c.nb - 1) {  // the sequence's last block may be partly filled
+    for (int r = 0; r < 4; ++r) s[r] = s4[r] * p.scale_log2e;
+    if (c.blk == c.nb - 1) {  // the sequence's last tile may be partly filled
       int ctx = p.context_lens[c.seq];
       ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
       const int tok0 = c.blk * BS;
       if (tok0 + BS > ctx) {
-        if (tok0 + tq >= ctx) {
 #pragma unroll
-          for (int g = 0; g < GT; ++g) s[g] = kNegInf;
-        }
+        for (int r = 0; r < 4; ++r) {
+          if (tok0 + kg + 4 * r >= ctx) {
+            s[r] = kNegInf;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i)
-          if (tok0 + i * RPL + rowg >= ctx) vv[i] = Vec16{{0u, 0u, 0u, 0u}};
-      }
-    }
-    // ---- lazy running maximum --------------------------------------------------
-    bool exceed = false;
-#pragma unroll
-    for (int g = 0; g < GT; ++g) exceed |= s[g] > m[g] + kLazyMaxSlack;
-    if (__any(exceed)) {  // wave-uniform, rare after a segment's first tile
-#pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        const float m_new = fmaxf(m[g], token_max(s[g]));
-        const float alpha = (m[g] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[g] - m_new);
-        l[g] *= alpha;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
-        m[g] = m_new;
-      }
-    }
-    // ---- probabilities -> LDS as 16-bit, grouped for the V-side rows -------------
-    float pr[GT];
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      const float ms = (m[g] == kNegInf) ? 0.f : m[g];
-      pr[g] = __builtin_amdgcn_exp2f(s[g] - ms);
-      l[g] += pr[g];
-    }
-#pragma unroll
-    for (int k = 0; k * 4 < GT; ++k) {  // lane qc writes heads qc, qc+4, ...
-      const float a0 = pr[4 * k];
-      const float a1 = 4 * k + 1 < GT ? pr[4 * k + 1] : 0.f;
-      const float a2 = 4 * k + 2 < GT ? pr[4 * k + 2] : 0.f;
-      const float a3 = 4 * k + 3 < GT ? pr[4 * k + 3] : 0.f;
-      const float lo = (qc & 1) ? a1 : a0;
-      const float hi = (qc & 1) ? a3 : a2;
-      const float mine = (qc & 2) ? hi : lo;
-      if (4 * k + qc < GT) s_p[wave][tq % RPL][4 * k + qc][tq / RPL] = E::narrow(mine);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- p.v: pack token pairs, one v_dot2 per (head, dim, pair) ------------------
-    // vv[i] holds token (i*RPL + rowg), dims col*8 .. col*8+7 as 4 packed dwords.
-    uint32_t lo01[4], hi01[4], lo23[4], hi23[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      lo01[k] = __builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x05040100u);
-      hi01[k] = __builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x07060302u);
-      if (NLD == 4) {
-        lo23[k] = __builtin_amdgcn_perm(vv[3 % NLD].w[k], vv[2 % NLD].w[k], 0x05040100u);
-        hi23[k] = __builtin_amdgcn_perm(vv[3 % NLD].w[k], vv[2 % NLD].w[k], 0x07060302u);
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      uint32_t p01, p23 = 0;
-      if (NLD == 4) {
-        const uint2 pp = *reinterpret_cast<const uint2 *>(&s_p[wave][rowg][g][0]);
-        p01 = pp.x;
-        p23 = pp.y;
-      } else {
-        p01 = *reinterpret_cast<const uint32_t *>(&s_p[wave][rowg][g][0]);
-      }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        acc[g][2 * k] = E::dot2(lo01[k], p01, acc[g][2 * k]);
-        acc[g][2 * k + 1] = E::dot2(hi01[k], p01, acc[g][2 * k + 1]);
-        if (NLD == 4) {
-          acc[g][2 * k] = E::dot2(lo23[k], p23, acc[g][2 * k]);
-          acc[g][2 * k + 1] = E::dot2(hi23[k], p23, acc[g][2 * k + 1]);
+            for (int k = 0; k < VW; ++k) vv[r].w[k] = 0u;
+          }
         }
       }
     }
-    // the slab is rewritten by the next tile
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    // ---- lazy running maximum ----------------------------------------------------
+    const float smax = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    if (__any(smax > m + kLazyMaxSlack)) {  // rare after a segment's first tile
+      float mx = smax;
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = (m == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float ar = __shfl(alpha, 4 * kg + r, kWave);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e][r] *= ar;
+      }
+    }
+    // ---- probabilities, rounded to the element type, as matrix A of p.v ----------
+    const float ms = (m == kNegInf) ? 0.f : m;
+    float pr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      pr[r] = __builtin_amdgcn_exp2f(s[r] - ms);
+      l += pr[r];
+    }
+    const Pair32 pa = {E::pack(pr[0], pr[1]), E::pack(pr[2], pr[3])};
+    // ---- p.v: token pairs packed per dim, one MFMA per dim of this lane -----------
+#pragma unroll
+    for (int k = 0; k < VW; ++k) {
+      const Pair32 even = {__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x05040100u),
+                           __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x05040100u)};
+      const Pair32 odd = {__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x07060302u),
+                          __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x07060302u)};
+      acc[2 * k] = E::pv(pa, even, acc[2 * k]);
+      acc[2 * k + 1] = E::pv(pa, odd, acc[2 * k + 1]);
+    }
     ++c.blk;
     --left;
     if (c.blk == c.nb || left == 0) finish_segment();
@@ -294,18 +279,19 @@ __global__ __launch_bounds__(NW *kWave) IC_GQA_OCC void paged_decode_gqa_kernel(
     uint32_t off_lo[SW], off_hi[SW];
     gather_window<BS, SW, ES>(p, lane, n_win, walk, off_lo, off_hi);
 
-    auto issue = [&](int i, Vec16 *kk, Vec16 *vv) {
+    auto issue = [&](int i, Vec16 *kk, VChunk<VW> *vv) {
       const int64_t tile = window_tile_offset(off_lo, off_hi, i);
       const char *kb = p.k_pool + tile;
       const char *vb = p.v_pool + tile;
 #pragma unroll
       for (int j = 0; j < NK; ++j) kk[j] = load16(kb + k_off[j]);
 #pragma unroll
-      for (int j = 0; j < NLD; ++j) vv[j] = load16(vb + v_off[j]);
+      for (int j = 0; j < NT; ++j) vv[j] = load_v<VW>(vb + v_off[j]);
       __builtin_amdgcn_sched_barrier(0);
     };
 
-    Vec16 ka[NK], va[NLD], kb[NK], vb[NLD];
+    Vec16 ka[NK], kb[NK];
+    VChunk<VW> va[NT], vb[NT];
     int i = 0;
     issue(0, ka, va);
     for (; i + 2 < n_win; i += 2) {
@@ -324,43 +310,29 @@ __global__ __launch_bounds__(NW *kWave) IC_GQA_OCC void paged_decode_gqa_kernel(
   }
 }
 
-template <class E, int HD, int GT>
+template <class E, int HD>
 bool launch_one(DecodeKP &kp, hipStream_t stream) {
   constexpr int BS = 16;
   constexpr int NW = kDecodeWavesPerWorkgroup;
   static const int per_cu = [] {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_gqa_kernel<E, HD, GT, BS, NW>,
-                                                     NW * kWave, 0) != hipSuccess || n < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_gqa_kernel<E, HD, BS, NW>, NW * kWave,
+                                                     0) != hipSuccess || n < 1)
       n = 1;
     return n;
   }();
   int wgs = per_cu * device_cu_count();
   if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
   kp.n_waves = wgs * NW;
-  hipLaunchKernelGGL((paged_decode_gqa_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
+  hipLaunchKernelGGL((paged_decode_gqa_kernel<E, HD, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
   return true;
 }
 
-template <class E, int HD>
-bool launch_gt(DecodeKP &kp, int gt, hipStream_t stream) {
-  switch (gt) {
-    case 2: return launch_one<E, HD, 2>(kp, stream);
-    case 3: return launch_one<E, HD, 3>(kp, stream);
-    case 4: return launch_one<E, HD, 4>(kp, stream);
-    case 5: return launch_one<E, HD, 5>(kp, stream);
-    case 6: return launch_one<E, HD, 6>(kp, stream);
-    case 7: return launch_one<E, HD, 7>(kp, stream);
-    case 8: return launch_one<E, HD, 8>(kp, stream);
-    default: return false;
-  }
-}
-
 template <class E>
-bool launch_hd(DecodeKP &kp, int hd, int gt, hipStream_t stream) {
+bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
   switch (hd) {
-    case 64: return launch_gt<E, 64>(kp, gt, stream);
-    case 128: return launch_gt<E, 128>(kp, gt, stream);
+    case 64: return launch_one<E, 64>(kp, stream);
+    case 128: return launch_one<E, 128>(kp, stream);
     default: return false;
   }
 }
@@ -368,9 +340,11 @@ bool launch_hd(DecodeKP &kp, int hd, int gt, hipStream_t stream) {
 }  // namespace
 
 bool launch_decode_gqa_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream) {
+  if (gt < 2 || gt > 16) return false;
+  kp.gt = gt;
   switch (dtype) {
-    case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, hd, gt, stream);
-    case IC_DTYPE_F16: return launch_hd<F16>(kp, hd, gt, stream);
+    case IC_DTYPE_BF16: return launch_hd<MfmaBf16>(kp, hd, stream);
+    case IC_DTYPE_F16: return launch_hd<MfmaF16>(kp, hd, stream);
     default: return false;
   }
 }
