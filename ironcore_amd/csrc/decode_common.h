@@ -84,11 +84,22 @@ __device__ __forceinline__ void next_pair(const DecodeKP &p, TileCursor &c) {
         c.nb = 0x7fffffff;
         return;
       }
-      c.nb = seq_blocks(p, c.seq, BS);
+      c.nb = __builtin_amdgcn_readfirstlane(seq_blocks(p, c.seq, BS));  // wave-uniform: keep it scalar
     } while (c.nb == 0);
   }
 }
 
+
+// Workgroups are dealt to the 8 XCDs round-robin by launch index.  Shares of
+// the tile sequence are handed out XCD-major instead, so that neighbouring
+// shares (sequences that may alias the same prefix blocks, and the query
+// sub-groups of one KV head) run on one XCD at the same time and meet in its
+// L2 instead of each fetching the blocks from HBM.
+__device__ __forceinline__ int xcd_major_workgroup() {
+  int wg = blockIdx.x;
+  if ((gridDim.x & 7) == 0) wg = (wg & 7) * (gridDim.x >> 3) + (wg >> 3);
+  return wg;
+}
 
 // This wave's share: [t0, t0 + left) of the batch-wide tile sequence and the
 // cursor of its first tile.  Every wave prefix-sums the per-sequence block

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   const int rowg = lane / LPR;
 
   // ---- this wave's share of the batch-wide tile sequence ----------------------
-  const int64_t wid = (int64_t)blockIdx.x * NW + wave;
+  const int64_t wid = (int64_t)xcd_major_workgroup() * NW + wave;
   int64_t left;  // tiles not yet consumed
   TileCursor c;
   if (!locate_chunk<BS>(p, lane, wid, left, c)) return;
@@ -287,43 +287,72 @@ constexpr int kReduceThreads = 256;
 // contiguous run of the batch-wide sequence, so the waves that touched it are
 // first_tile / chunk .. last_tile / chunk and their partial ids follow.
 // Traffic is (hd+2)*4 bytes per partial, three orders of magnitude below the
-// K/V stream.
+// K/V stream; what costs time here is the chain of dependent memory round
+// trips, so the prefix sums are fetched together and every thread fetches up
+// to four partials of its four output dims in one batch before it merges them
+// (a typical pair has two to four partials: two round trips in all).
 template <class E, int HD, int GT>
 __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(const DecodeKP p) {
   using T = typename E::type;
+  constexpr int QPH = HD / 4;  // 4-dim groups per head row
+  constexpr int UB = 4;        // partials fetched per batch
   const int pair_in_seq = blockIdx.x;
   const int seq = blockIdx.y;
+  const int cum = p.cum_blocks[seq];
+  const int cum_next = p.cum_blocks[seq + 1];
+  const int cum_all = p.cum_blocks[p.n_seqs];
   const int kvh = pair_in_seq / p.nsub;
   const int sub = pair_in_seq - kvh * p.nsub;
   const int head0 = kvh * p.group + sub * GT;
   const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
   T *orow = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)head0 * HD;
-  const int cum = p.cum_blocks[seq];
-  const int nb = p.cum_blocks[seq + 1] - cum;
+  const int nb = cum_next - cum;
   if (nb == 0) {  // no visible token: zero rows
     for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) orow[o] = E::narrow(0.f);
     return;
   }
-  const int64_t n_tiles = (int64_t)p.cum_blocks[p.n_seqs] * p.pairs_per_seq;
+  const int64_t n_tiles = (int64_t)cum_all * p.pairs_per_seq;
   const int64_t chunk = chunk_tiles(p, n_tiles);
   const int64_t first = (int64_t)cum * p.pairs_per_seq + (int64_t)pair_in_seq * nb;
   const int64_t w0 = first / chunk;
   const int64_t w1 = (first + nb - 1) / chunk;
   if (w0 == w1) return;  // one wave covered the whole pair and wrote the rows
   const int64_t base = (int64_t)seq * p.pairs_per_seq + pair_in_seq;
-  for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) {
-    const int g = o / HD;
-    const int d = o - g * HD;
-    float mx = kNegInf;
-    for (int64_t w = w0; w <= w1; ++w) mx = fmaxf(mx, p.part_ml[((w + base) * GT + g) * 2]);
-    float lsum = 0.f, a = 0.f;
-    for (int64_t w = w0; w <= w1; ++w) {
-      const int64_t slot = (w + base) * GT + g;
-      const float wt = __builtin_amdgcn_exp2f(p.part_ml[slot * 2] - mx);
-      lsum = __builtin_fmaf(p.part_ml[slot * 2 + 1], wt, lsum);
-      a = __builtin_fmaf(p.part_acc[slot * HD + d], wt, a);
+  for (int o = threadIdx.x; o < heads * QPH; o += kReduceThreads) {
+    const int g = o / QPH;
+    const int d = (o - g * QPH) * 4;
+    float m_run = kNegInf, l_run = 0.f;
+    float4 a_run = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int64_t wb = w0; wb <= w1; wb += UB) {
+      float2 ml[UB];
+      float4 av[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {  // independent loads, all in flight together
+        const int64_t w = wb + u <= w1 ? wb + u : w1;
+        const int64_t slot = (w + base) * GT + g;
+        ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
+        av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
+      }
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        if (wb + u > w1 || ml[u].x == kNegInf) continue;
+        const float m_new = fmaxf(m_run, ml[u].x);
+        const float keep = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float wt = __builtin_amdgcn_exp2f(ml[u].x - m_new);
+        l_run = __builtin_fmaf(ml[u].y, wt, l_run * keep);
+        a_run.x = __builtin_fmaf(av[u].x, wt, a_run.x * keep);
+        a_run.y = __builtin_fmaf(av[u].y, wt, a_run.y * keep);
+        a_run.z = __builtin_fmaf(av[u].z, wt, a_run.z * keep);
+        a_run.w = __builtin_fmaf(av[u].w, wt, a_run.w * keep);
+        m_run = m_new;
+      }
     }
-    orow[o] = E::narrow(a / lsum);
+    const float inv = 1.f / l_run;
+    T *dst = orow + g * HD + d;
+    dst[0] = E::narrow(a_run.x * inv);
+    dst[1] = E::narrow(a_run.y * inv);
+    dst[2] = E::narrow(a_run.z * inv);
+    dst[3] = E::narrow(a_run.w * inv);
   }
 }
 

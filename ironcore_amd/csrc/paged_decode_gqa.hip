@@ -113,10 +113,16 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_gqa_kernel(const Decod
   const int n = lane & 15;   // matrix column: head (q.k) or dim group (p.v)
   const int kg = lane >> 4;  // this lane's tokens are kg, kg+4, kg+8, kg+12
 
-  const int64_t wid = (int64_t)blockIdx.x * NW + wave;
-  int64_t left;
+  const int64_t wid = (int64_t)xcd_major_workgroup() * NW + wave;
+  int64_t left64;
   TileCursor c;
-  if (!locate_chunk<BS>(p, lane, wid, left, c)) return;
+  if (!locate_chunk<BS>(p, lane, wid, left64, c)) return;
+  // wave-uniform by construction; say so, so the bookkeeping is scalar work
+  c.seq = __builtin_amdgcn_readfirstlane(c.seq);
+  c.pair = __builtin_amdgcn_readfirstlane(c.pair);
+  c.blk = __builtin_amdgcn_readfirstlane(c.blk);
+  c.nb = __builtin_amdgcn_readfirstlane(c.nb);
+  int left = __builtin_amdgcn_readfirstlane((int)left64);
   TileCursor walk = c;
   TileCursor peek = c;
   next_pair<BS>(p, peek);
@@ -219,7 +225,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_gqa_kernel(const Decod
 #pragma unroll
     for (int r = 0; r < 4; ++r) s[r] = s4[r] * p.scale_log2e;
     if (c.blk == c.nb - 1) {  // the sequence's last tile may be partly filled
-      int ctx = p.context_lens[c.seq];
+      int ctx = __builtin_amdgcn_readfirstlane(p.context_lens[c.seq]);
       ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
       const int tok0 = c.blk * BS;
       if (tok0 + BS > ctx) {
@@ -275,7 +281,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_gqa_kernel(const Decod
   };
 
   while (left > 0) {
-    const int n_win = left < kWave * SW ? (int)left : kWave * SW;
+    const int n_win = left < kWave * SW ? left : kWave * SW;
     uint32_t off_lo[SW], off_hi[SW];
     gather_window<BS, SW, ES>(p, lane, n_win, walk, off_lo, off_hi);
 
