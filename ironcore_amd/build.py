@@ -20,7 +20,7 @@ LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libironcore_paged.so"
 OBJ_DIR = PKG / "build" / "obj"
 
-SOURCES = ["ic_api.hip", "kv_append.hip", "paged_decode.hip", "paged_decode_gqa.hip", "paged_prefill.hip"]
+SOURCES = ["ic_api.hip", "kv_append.hip", "paged_decode.hip", "paged_decode_mfma.hip", "paged_prefill.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -46,7 +46,7 @@ def _hipcc() -> str:
 # VGPRs: the softmax rescales them with VALU instructions, and the AGPR form
 # costs a register copy each way per tile.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
-PER_SOURCE_FLAGS = {"paged_prefill.hip": _VGPR_FORM, "paged_decode_gqa.hip": _VGPR_FORM}
+PER_SOURCE_FLAGS = {"paged_prefill.hip": _VGPR_FORM, "paged_decode_mfma.hip": _VGPR_FORM}
 
 
 def _compile(src: str, extra: list[str]) -> Path:

@@ -223,9 +223,9 @@ __device__ __forceinline__ int64_t window_tile_offset(const uint32_t *off_lo, co
 
 constexpr int kDecodeWavesPerWorkgroup = 4;
 
-// Launches the query-group decode main kernel (paged_decode_gqa.hip) when it is
+// Launches the query-group decode main kernel (paged_decode_mfma.hip) when it is
 // built for this shape; returns false otherwise.  Sets kp.n_waves.
-bool launch_decode_gqa_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream);
+bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream);
 
 }  // namespace decode
 }  // namespace ic

@@ -3,8 +3,13 @@
 // What it computes is the reference's dense attention with sq = 1
 // (ironcore/layers/attention.py:68-142) on the rows the block table names:
 // scores = q.k * scale, softmax over the context, out = probs @ v, with query
-// head h reading KV head h / G (attention.py:95-102).  Scores, softmax and the
-// PV sum stay in fp32; only the result is rounded to the element type.
+// head h reading KV head h / G (attention.py:95-102).
+//
+// This file holds the host-side launch, the split-K reduce pass and the
+// vector-ALU main kernel, which is the one fp32 pools run on (scores, softmax
+// and the PV sum stay in fp32).  bf16 and fp16 pools take the matrix-core main
+// kernel of paged_decode_mfma.hip; both share everything described here
+// except the arithmetic of a tile.
 //
 // HBM-bound streaming kernel (one pass over every visible K and V byte).
 //
@@ -20,7 +25,8 @@
 //    span several pairs; each (wave, pair) segment yields one partial.  All
 //    waves carry the same load whatever the spread of context lengths, the
 //    grid is exactly the number of waves the GPU holds at once, and waves
-//    never synchronise with each other.
+//    never synchronise with each other.  Shares are dealt XCD-major, so
+//    neighbouring shares (which may alias the same prefix blocks) share an L2.
 //  * At the start of its chunk a wave gathers the byte offsets of its next
 //    256 tiles from the block table, one per lane and slot; the loop reads
 //    them back as wave-uniform scalars (v_readlane), so the table is off the
@@ -31,9 +37,10 @@
 //    register tiles in ping-pong: the next tile's loads are in flight while
 //    the current one is consumed, across pair boundaries too; the next
 //    pair's query is prefetched a segment ahead.
-//  * q.k: v_dot2 on the packed pairs, then a DPP butterfly over the LPR lanes
-//    that share a row.  Online softmax per lane group; p*v accumulates into
-//    EPL fp32 registers per query head with no cross-lane traffic.
+//  * q.k: fused multiply-adds (v_dot2 for 16-bit types), then a DPP butterfly
+//    over the LPR lanes that share a row.  Online softmax per lane group; p*v
+//    accumulates into EPL fp32 registers per query head with no cross-lane
+//    traffic.
 //  * Segment end: the lane groups of the wave are merged (log-sum-exp) through
 //    a private LDS slab.  A segment that covers its whole pair writes the
 //    output row; otherwise (m, l, acc) go to the workspace and the reduce
@@ -373,8 +380,10 @@ template <class E, int HD, int GT>
 int launch_typed(DecodeKP &kp, int dtype, hipStream_t stream) {
   constexpr int BS = 16;
   constexpr int NW = kDecodeWavesPerWorkgroup;
-  // Several query heads per KV head: the query-group kernel (16-bit types).
-  if (!(GT > 1 && launch_decode_gqa_main(kp, dtype, HD, GT, stream))) {
+  if constexpr (sizeof(typename E::type) == 2) {
+    // 16-bit element types: the matrix-core kernel, whatever the group size.
+    if (!launch_decode_mfma_main(kp, dtype, HD, GT, stream)) return IC_ERR_UNSUPPORTED;
+  } else {
     int wgs = resident_workgroups<E, HD, GT, BS, NW>();
     if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
     kp.n_waves = wgs * NW;

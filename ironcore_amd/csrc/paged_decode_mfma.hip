@@ -1,5 +1,5 @@
-// Paged decode for grouped-query attention (several query heads per KV head),
-// 16-bit element types, on the matrix cores.
+// Paged decode main kernel for 16-bit element types (bf16, fp16), on the
+// matrix cores, for any number G of query heads per KV head (1 .. 8 per wave).
 //
 // Same result, same balanced split-K bookkeeping, same partial format and
 // reduce pass as paged_decode.hip.  What changes is the arithmetic of a tile:
@@ -19,7 +19,8 @@
 //    token's K row), so lane l owns tokens kg, kg+4, kg+8, kg+12 (kg = l/16):
 //    exactly the four k-elements lane l must supply for matrix A of the next
 //    product.  exp2 and the 16-bit rounding (the reference rounds the
-//    probabilities to the element type too) happen in place.
+//    probabilities to the element type too, attention.py:124-134) happen in
+//    place.
 //  * O += P . V    (v_mfma_f32_16x16x16, one per dim owned by a lane).  B = V:
 //    lane l loads dims (l%16)*hd/16 .. of tokens kg + 4i (coalesced rows) and
 //    packs token pairs with v_perm_b32; MFMA e covers dim (l%16)*hd/16 + e.
@@ -30,7 +31,7 @@
 //    folded once per segment.
 //
 // Per tile and wave: hd/32 + hd/16 MFMAs and about 50 vector instructions,
-// whatever G is.
+// whatever G is, which leaves the kernel bound by HBM alone.
 #include "decode_common.h"
 #include "../../include/ironcore_paged.h"
 
@@ -98,7 +99,7 @@ __device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
 }
 
 template <class E, int HD, int BS, int NW>
-__global__ __launch_bounds__(NW *kWave) void paged_decode_gqa_kernel(const DecodeKP p) {
+__global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int ES = 2;
   constexpr int NK = HD / 32;  // q.k MFMAs = 16-byte K loads per lane per tile
@@ -322,7 +323,7 @@ bool launch_one(DecodeKP &kp, hipStream_t stream) {
   constexpr int NW = kDecodeWavesPerWorkgroup;
   static const int per_cu = [] {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_gqa_kernel<E, HD, BS, NW>, NW * kWave,
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_mfma_kernel<E, HD, BS, NW>, NW * kWave,
                                                      0) != hipSuccess || n < 1)
       n = 1;
     return n;
@@ -330,7 +331,7 @@ bool launch_one(DecodeKP &kp, hipStream_t stream) {
   int wgs = per_cu * device_cu_count();
   if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
   kp.n_waves = wgs * NW;
-  hipLaunchKernelGGL((paged_decode_gqa_kernel<E, HD, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
+  hipLaunchKernelGGL((paged_decode_mfma_kernel<E, HD, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
   return true;
 }
 
@@ -345,8 +346,8 @@ bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
 
 }  // namespace
 
-bool launch_decode_gqa_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream) {
-  if (gt < 2 || gt > 16) return false;
+bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream) {
+  if (gt < 1 || gt > 16) return false;
   kp.gt = gt;
   switch (dtype) {
     case IC_DTYPE_BF16: return launch_hd<MfmaBf16>(kp, hd, stream);
