@@ -49,6 +49,8 @@ def parse():
     ap.add_argument("--layers", type=int, default=4, help="resident layer pools the steps rotate over")
     ap.add_argument("--min-chunk-tokens", type=int, default=0, help="smallest split-K share (0 = library default)")
     ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo", "prefill"])
+    ap.add_argument("--cohort-size", type=int, default=0,
+                    help="shared-prefix cohort size for decode (0 = 2 when the workload aliases prefixes, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
     ap.add_argument("--seed", type=int, default=0)
@@ -112,6 +114,14 @@ def bench_decode(args, torch, dev):
     k_new = torch.randn(b, gn, hd, generator=g, device=dev, dtype=torch.float32).to(wl.k_pool.dtype)
     v_new = torch.randn(b, gn, hd, generator=g, device=dev, dtype=torch.float32).to(wl.k_pool.dtype)
     out = torch.empty(b, hn * hd, dtype=wl.query.dtype, device=dev)
+    # sequences that alias prefix blocks (GRPO samples of one prompt) are decoded in
+    # cohorts that stream the shared blocks once; the sharing is a property of the
+    # block tables, found on the host once, outside the timed region
+    cohort = args.cohort_size if args.cohort_size > 0 else (2 if wl.logical_tokens != wl.unique_tokens else 1)
+    shared = None
+    if cohort > 1:
+        shared = torch.from_numpy(paged_ops.shared_prefix_blocks(
+            wl.block_tables.cpu().numpy(), wl.context_lens.cpu().numpy(), bs, cohort)).to(dev)
 
     def step(i, ev):
         kp, vp = pools[i % len(pools)]
@@ -119,7 +129,8 @@ def bench_decode(args, torch, dev):
         if ev:
             ev[0].record()
         paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
-                               wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens)
+                               wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens,
+                               cohort_size=cohort, cohort_shared_blocks=shared)
         if ev:
             ev[1].record()
 
@@ -152,13 +163,13 @@ def bench_decode(args, torch, dev):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl.name, "batch": b, "q_heads": hn, "kv_heads": gn, "head_dim": hd,
                    "block_size": bs, "sum_context": wl.logical_tokens, "unique_tokens": wl.unique_tokens,
-                   "resident_layers": len(pools),
+                   "resident_layers": len(pools), "cohort_size": cohort,
                    "step": f"kv_append({b} rows) + paged_decode, one layer"},
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.seed)),
-                     "kernel": "paged_decode_kernel (+ split-K reduce)",
+                     "kernel": "paged_decode_mfma_kernel (+ paged_decode_reduce_kernel)",
                      "bytes_per_launch": decode_bytes, "avg_launch_ms": round(decode_ms_avg, 5),
                      "median_launch_ms": round(statistics.median(decode_ms), 5)},
     }

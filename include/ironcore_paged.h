@@ -103,7 +103,8 @@ size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd);
  * sq = 1 on the rows the block table points at:
  *     out[i, h*hd + d] = sum_j softmax_j(q[i,h] . k[i,j,h/G] * scale) * v[i,j,h/G,d]
  *
- *   out           [n_seqs, hn*hd], row stride out_stride_seq
+ *   out           [n_seqs, hn*hd], row stride out_stride_seq (16-byte aligned
+ *                 rows for bf16 / fp16)
  *   q             [n_seqs, hn, hd], row stride q_stride_seq
  *   scale         multiplies q.k (the reference divides by sqrt(hd),
  *                 attention.py:65,110; pass 1/sqrt(hd))
@@ -128,6 +129,46 @@ int ic_paged_decode(void *out, int64_t out_stride_seq,
                     int64_t num_blocks, int max_context_len, float scale,
                     int min_chunk_tokens, void *workspace, size_t workspace_bytes,
                     int dtype, void *stream);
+
+/*
+ * Paged decode for batches whose sequences alias prefix blocks (sampling
+ * several continuations of one prompt: the block tables of a group repeat the
+ * prompt's blocks, as a fork of the block KV cache leaves them).  Same result
+ * as ic_paged_decode on the same arguments; the aliased blocks are streamed
+ * from HBM once per cohort instead of once per sequence.  The reference has
+ * no counterpart (it has no KV cache; every sample recomputes its prompt,
+ * examples/generate_text.py:27); the attention it must reproduce is still
+ * ironcore/layers/attention.py:68-142.
+ *
+ *   cohort_size           S >= 1: sequences i*S .. i*S+S-1 of the batch form
+ *                         cohort i (the last one may be short).  1 = no
+ *                         sharing, identical to ic_paged_decode.
+ *                         (hn / gn) * S must not exceed 32; bf16 / fp16 only.
+ *   cohort_shared_blocks  int32 [ceil(n_seqs / S)]: for each cohort, how many
+ *                         leading block-table entries are the SAME pool block
+ *                         in all its members' rows.  May under-state the
+ *                         sharing (0 is always valid); must not over-state it.
+ *                         Only blocks every member's context covers entirely
+ *                         are treated as shared.  Ignored (may be NULL) when
+ *                         cohort_size is 1.
+ *   workspace             at least ic_paged_decode_shared_workspace_bytes(...)
+ * Everything else as for ic_paged_decode.
+ */
+size_t ic_paged_decode_shared_workspace_bytes(int n_seqs, int hn, int gn, int hd,
+                                              int cohort_size);
+int ic_paged_decode_shared(void *out, int64_t out_stride_seq,
+                           const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool,
+                           int64_t pool_stride_block, int64_t pool_stride_head,
+                           int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens,
+                           int n_seqs, int hn, int gn, int hd, int block_size,
+                           int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens,
+                           int cohort_size, const int32_t *cohort_shared_blocks,
+                           void *workspace, size_t workspace_bytes,
+                           int dtype, void *stream);
 
 /*
  * Chunked prefill against the block KV cache: each sequence brings a chunk of

@@ -30,13 +30,23 @@ struct DecodeKP {
   int hn;
   int group;        // query heads per KV head
   int nsub;         // query sub-groups per KV head (ceil(group / GT))
-  int gt;           // query heads per sub-group (the stride of the partial arrays)
+  int gt;           // matrix columns per pair = query heads per sub-group, times the
+                    // cohort size with cohorts (the stride of the partial arrays)
   int pairs_per_seq;  // gn * nsub
   int max_ctx;
   int n_waves;      // waves in the main kernel's grid
   int min_chunk;    // smallest chunk, in tiles
   int tiles_per_block;  // 16-token tiles in one pool block (1 for block_size 16)
   float scale_log2e;
+  // Shared-prefix cohorts (matrix-core kernel only).  cohort_size consecutive
+  // sequences form a cohort whose first cohort_shared[c] pool blocks are the
+  // same physical blocks; those tiles are streamed once for the whole cohort.
+  // Work is laid out in ROWS: with cohort_size 1 a row is a sequence; otherwise
+  // cohort c owns rows c*(S+1) .. c*(S+1)+S: the shared tiles (all members'
+  // heads as matrix columns), then each member's private tiles.
+  const int32_t *cohort_shared;  // [ceil(n_seqs / cohort_size)] pool blocks, or nullptr
+  int cohort_size;               // S >= 1
+  int n_rows;                    // n_seqs, or n_cohorts * (S + 1)
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
@@ -45,6 +55,43 @@ __device__ __forceinline__ int seq_blocks(const DecodeKP &p, int seq, int bs) {
   int ctx = p.context_lens[seq];
   ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
   return ctx > 0 ? (ctx + bs - 1) / bs : 0;
+}
+
+// Tiles of cohort c that are streamed once for all members: the caller's
+// count of aliased blocks, cut down to whole tiles every member's context
+// covers (so a shared tile never needs a mask).
+__device__ __forceinline__ int cohort_shared_tiles(const DecodeKP &p, int c) {
+  int sh = p.cohort_shared[c] * p.tiles_per_block;
+  for (int u = 0; u < p.cohort_size; ++u) {
+    const int s = c * p.cohort_size + u;
+    if (s >= p.n_seqs) break;
+    int ctx = p.context_lens[s];
+    ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
+    const int whole = ctx > 0 ? ctx / 16 : 0;
+    sh = sh < whole ? sh : whole;
+  }
+  return sh > 0 ? sh : 0;
+}
+
+// A row of the work layout: which sequence's block table it walks, its
+// first tile in that sequence and how many tiles it has.
+struct RowSpan {
+  int tseq;   // sequence whose block-table row addresses the tiles
+  int first;  // first tile (of the sequence) in this row
+  int tiles;
+};
+
+template <int BS>
+__device__ __forceinline__ RowSpan row_span(const DecodeKP &p, int row) {
+  if (p.cohort_size == 1) return RowSpan{row, 0, seq_blocks(p, row, BS)};
+  const int rpc = p.cohort_size + 1;
+  const int c = row / rpc;
+  const int j = row - c * rpc;
+  const int sh = cohort_shared_tiles(p, c);
+  if (j == 0) return RowSpan{c * p.cohort_size, 0, sh};
+  const int s = c * p.cohort_size + j - 1;
+  if (s >= p.n_seqs) return RowSpan{p.n_seqs - 1, 0, 0};
+  return RowSpan{s, sh, seq_blocks(p, s, BS) - sh};
 }
 
 // Tiles per wave: equal shares of the N tiles, never below min_chunk.
@@ -63,14 +110,23 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
   return v;
 }
 
-// Position in the batch-wide tile sequence: block `blk` of pair
-// (seq, pair) whose sequence has `nb` blocks.  Wave-uniform.
+// Position in the batch-wide tile sequence: tile `blk` of pair (row, pair)
+// whose row has `nb` tiles.  Wave-uniform.
 struct TileCursor {
-  int seq;
+  int seq;    // row (= sequence when there are no cohorts)
   int pair;
   int blk;
   int nb;
+  int tseq;   // block-table row of this row's tiles
+  int first;  // tile of that sequence the row starts at
 };
+
+__device__ __forceinline__ void set_row(TileCursor &c, int row, const RowSpan &r) {
+  c.seq = row;
+  c.nb = __builtin_amdgcn_readfirstlane(r.tiles);  // wave-uniform: keep it scalar
+  c.tseq = __builtin_amdgcn_readfirstlane(r.tseq);
+  c.first = __builtin_amdgcn_readfirstlane(r.first);
+}
 
 template <int BS>
 __device__ __forceinline__ void next_pair(const DecodeKP &p, TileCursor &c) {
@@ -79,16 +135,15 @@ __device__ __forceinline__ void next_pair(const DecodeKP &p, TileCursor &c) {
     c.pair = 0;
     do {
       ++c.seq;
-      if (c.seq >= p.n_seqs) {  // past the last tile: never dereferenced
-        c.seq = p.n_seqs;
+      if (c.seq >= p.n_rows) {  // past the last tile: never dereferenced
+        c.seq = p.n_rows;
         c.nb = 0x7fffffff;
         return;
       }
-      c.nb = __builtin_amdgcn_readfirstlane(seq_blocks(p, c.seq, BS));  // wave-uniform: keep it scalar
+      set_row(c, c.seq, row_span<BS>(p, c.seq));
     } while (c.nb == 0);
   }
 }
-
 
 // Workgroups are dealt to the 8 XCDs round-robin by launch index.  Shares of
 // the tile sequence are handed out XCD-major instead, so that neighbouring
@@ -102,48 +157,85 @@ __device__ __forceinline__ int xcd_major_workgroup() {
 }
 
 // This wave's share: [t0, t0 + left) of the batch-wide tile sequence and the
-// cursor of its first tile.  Every wave prefix-sums the per-sequence block
-// counts itself (64 sequences per step, one per lane): first for the total,
-// which fixes the chunk size, then again to find the sequence that holds its
-// first tile.  Wave 0 also leaves the prefix sums in the workspace for the
-// reduce kernel.  Returns false when the wave has no tiles.
+// cursor of its first tile.  Every wave prefix-sums the per-row tile counts
+// itself (kRowsPerLane consecutive rows per lane and step, their loads in
+// flight together): first for the total, which fixes the chunk size, then
+// again to find the row that holds its first tile.  Wave 0 also leaves the
+// prefix sums in the workspace for the reduce kernel.  Returns false when the
+// wave has no tiles.
+constexpr int kRowsPerLane = 4;
+
 template <int BS>
 __device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int64_t wid, int64_t &left,
                                              TileCursor &c) {
-  int64_t total_blocks = 0;
-  for (int base = 0; base < p.n_seqs; base += kWave) {
-    const int s = base + lane;
-    const int mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
+  constexpr int RPS = kWave * kRowsPerLane;  // rows per step
+  int64_t total = 0;
+  for (int base = 0; base < p.n_rows; base += RPS) {
+    int cnt[kRowsPerLane];
+#pragma unroll
+    for (int k = 0; k < kRowsPerLane; ++k) {
+      const int r = base + lane * kRowsPerLane + k;
+      cnt[k] = r < p.n_rows ? row_span<BS>(p, r).tiles : 0;
+    }
+    int mine = 0;
+#pragma unroll
+    for (int k = 0; k < kRowsPerLane; ++k) mine += cnt[k];
     const int incl = wave_inclusive_scan(mine, lane);
-    if (wid == 0 && s < p.n_seqs) p.cum_blocks[s + 1] = (int32_t)(total_blocks + incl);
-    total_blocks += __builtin_amdgcn_readlane(incl, kWave - 1);
+    if (wid == 0) {
+      int run = (int)total + incl - mine;
+#pragma unroll
+      for (int k = 0; k < kRowsPerLane; ++k) {
+        const int r = base + lane * kRowsPerLane + k;
+        run += cnt[k];
+        if (r < p.n_rows) p.cum_blocks[r + 1] = run;
+      }
+    }
+    total += __builtin_amdgcn_readlane(incl, kWave - 1);
   }
   if (wid == 0 && lane == 0) p.cum_blocks[0] = 0;
-  const int64_t n_tiles = total_blocks * p.pairs_per_seq;
+  const int64_t n_tiles = total * p.pairs_per_seq;
   const int64_t chunk = chunk_tiles(p, n_tiles);
   const int64_t t0 = wid * chunk;
   if (t0 >= n_tiles) return false;
   left = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;
 
-  int64_t before = 0;  // blocks of the sequences scanned so far
-  c.seq = p.n_seqs;
-  c.nb = 1;
+  int64_t before = 0;  // tiles of the rows scanned so far
+  int row = p.n_rows;
   int cum = 0;
-  for (int base = 0; base < p.n_seqs; base += kWave) {
-    const int s = base + lane;
-    const int mine = s < p.n_seqs ? seq_blocks(p, s, BS) : 0;
+  for (int base = 0; base < p.n_rows; base += RPS) {
+    int cnt[kRowsPerLane];
+#pragma unroll
+    for (int k = 0; k < kRowsPerLane; ++k) {
+      const int r = base + lane * kRowsPerLane + k;
+      cnt[k] = r < p.n_rows ? row_span<BS>(p, r).tiles : 0;
+    }
+    int mine = 0;
+#pragma unroll
+    for (int k = 0; k < kRowsPerLane; ++k) mine += cnt[k];
     const int incl = wave_inclusive_scan(mine, lane);
-    // first sequence whose tiles end after t0
+    // first lane whose rows end after t0
     const uint64_t hit = __ballot((before + incl) * p.pairs_per_seq > t0);
     if (hit != 0) {
       const int ln = __builtin_ctzll(hit);
-      c.seq = base + ln;
-      c.nb = __builtin_amdgcn_readlane(mine, ln);
-      cum = (int)(before + __builtin_amdgcn_readlane(incl, ln)) - c.nb;
+      int run = (int)before + __builtin_amdgcn_readlane(incl - mine, ln);
+      int found = -1, found_cum = 0;
+#pragma unroll
+      for (int k = 0; k < kRowsPerLane; ++k) {
+        const int n = __builtin_amdgcn_readlane(cnt[k], ln);
+        if (found < 0 && (int64_t)(run + n) * p.pairs_per_seq > t0) {
+          found = k;
+          found_cum = run;
+        }
+        run += n;
+      }
+      row = base + ln * kRowsPerLane + found;
+      cum = found_cum;
       break;
     }
     before += __builtin_amdgcn_readlane(incl, kWave - 1);
   }
+  row = __builtin_amdgcn_readfirstlane(row);
+  set_row(c, row, row_span<BS>(p, row));
   const int64_t r = t0 - (int64_t)cum * p.pairs_per_seq;
   c.pair = (int)(r / c.nb);
   c.blk = (int)(r - (int64_t)c.pair * c.nb);
@@ -167,12 +259,12 @@ __device__ __forceinline__ void gather_window(const DecodeKP &p, int lane, int n
   for (int pos = 0; pos < n_win;) {  // wave-uniform walk over the window's segments
     const int cnt = (walk.nb - walk.blk < n_win - pos) ? walk.nb - walk.blk : n_win - pos;
     const int kvh = walk.pair / p.nsub;
-    const int64_t row = (int64_t)walk.seq * p.bt_stride;
+    const int64_t row = (int64_t)walk.tseq * p.bt_stride;
 #pragma unroll
     for (int r = 0; r < SW; ++r) {
       const int lp = r * kWave + lane;
       const bool in = lp >= pos && lp < pos + cnt;
-      int tile_in_seq = walk.blk + lp - pos;
+      int tile_in_seq = walk.first + walk.blk + lp - pos;
       int sub = 0;
       if (p.tiles_per_block > 1) {  // pool blocks longer than one tile
         const int b = tile_in_seq / p.tiles_per_block;
@@ -223,9 +315,10 @@ __device__ __forceinline__ int64_t window_tile_offset(const uint32_t *off_lo, co
 
 constexpr int kDecodeWavesPerWorkgroup = 4;
 
-// Launches the query-group decode main kernel (paged_decode_mfma.hip) when it is
-// built for this shape; returns false otherwise.  Sets kp.n_waves.
-bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream);
+// Launches the matrix-core decode main kernel (paged_decode_mfma.hip) when it
+// is built for this shape (16-bit dtype, hd 64 or 128, kp.gt <= 32 columns);
+// returns false otherwise.  Sets kp.n_waves.
+bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream);
 
 }  // namespace decode
 }  // namespace ic

@@ -96,8 +96,13 @@ int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
 }
 
 size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd) {
-  if (n_seqs <= 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0) return 0;
-  return ic::decode_workspace(n_seqs, hn, gn, hd).total();
+  return ic_paged_decode_shared_workspace_bytes(n_seqs, hn, gn, hd, 1);
+}
+
+size_t ic_paged_decode_shared_workspace_bytes(int n_seqs, int hn, int gn, int hd, int cohort_size) {
+  if (n_seqs <= 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0 || cohort_size < 1) return 0;
+  if (cohort_size > 1 && (hn / gn) * cohort_size > ic::kMaxCohortColumns) return 0;
+  return ic::decode_workspace(n_seqs, hn, gn, hd, cohort_size).total();
 }
 
 int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
@@ -107,7 +112,23 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
                     int gn, int hd, int block_size, int64_t num_blocks, int max_context_len,
                     float scale, int min_chunk_tokens, void *workspace, size_t workspace_bytes,
                     int dtype, void *stream) {
-  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0) return IC_ERR_BAD_SHAPE;
+  return ic_paged_decode_shared(out, out_stride_seq, q, q_stride_seq, k_pool, v_pool, pool_stride_block,
+                                pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                                context_lens, n_seqs, hn, gn, hd, block_size, num_blocks,
+                                max_context_len, scale, min_chunk_tokens, 1, nullptr, workspace,
+                                workspace_bytes, dtype, stream);
+}
+
+int ic_paged_decode_shared(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                           int64_t pool_stride_head, int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens, int n_seqs, int hn, int gn, int hd,
+                           int block_size, int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens, int cohort_size, const int32_t *cohort_shared_blocks,
+                           void *workspace, size_t workspace_bytes, int dtype, void *stream) {
+  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0 || cohort_size < 1)
+    return IC_ERR_BAD_SHAPE;
   if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
   const int es = ic::elem_size(dtype);
   if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
@@ -115,6 +136,10 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
     return rc;
   if (n_seqs == 0) return IC_OK;
   if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
+  if (cohort_size > 1) {
+    if (!cohort_shared_blocks) return IC_ERR_NULL_POINTER;
+    if (dtype == IC_DTYPE_F32 || (hn / gn) * cohort_size > ic::kMaxCohortColumns) return IC_ERR_UNSUPPORTED;
+  }
   if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
   if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
   const int mc = resolve_min_chunk(min_chunk_tokens);
@@ -123,7 +148,9 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
   if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;
   if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !stride16(q_stride_seq, es))
     return IC_ERR_ALIGNMENT;
-  const ic::DecodeWorkspace ws = ic::decode_workspace(n_seqs, hn, gn, hd);
+  // the matrix-core kernel stores 8- or 16-byte pieces of output rows
+  if (es == 2 && (!aligned16(out) || !stride16(out_stride_seq, es))) return IC_ERR_ALIGNMENT;
+  const ic::DecodeWorkspace ws = ic::decode_workspace(n_seqs, hn, gn, hd, cohort_size);
   if (!workspace || workspace_bytes < ws.total() || (reinterpret_cast<uintptr_t>(workspace) & 255u))
     return IC_ERR_WORKSPACE;
 
@@ -149,6 +176,8 @@ int ic_paged_decode(void *out, int64_t out_stride_seq, const void *q, int64_t q_
   a.cum_blocks = reinterpret_cast<int32_t *>(wsp);
   a.part_ml = reinterpret_cast<float *>(wsp + ws.cum_bytes);
   a.part_acc = reinterpret_cast<float *>(wsp + ws.cum_bytes + ws.ml_bytes);
+  a.cohort_size = cohort_size;
+  a.cohort_shared_blocks = cohort_shared_blocks;
   a.dtype = dtype;
   return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
 }

@@ -48,9 +48,11 @@ struct DecodeArgs {
   int max_context_len;
   float scale;
   int min_chunk_tokens;  // smallest split-K share (multiple of block_size)
-  int32_t *cum_blocks;   // workspace: [n_seqs + 1]
+  int32_t *cum_blocks;   // workspace: [rows + 1]
   float *part_ml;        // workspace: [partial slots, 2]
   float *part_acc;       // workspace: [partial slots, hd]
+  int cohort_size;       // 1 = no shared prefixes
+  const int32_t *cohort_shared_blocks;  // [ceil(n_seqs / cohort_size)], or nullptr
   int dtype;
 };
 
@@ -93,21 +95,38 @@ inline int elem_size(int dtype) { return dtype == 2 ? 4 : 2; }
 // groups are cut into ceil(group / 8) sub-groups.
 inline int decode_heads_per_wave(int group) { return group <= 8 ? group : 8; }
 
-// Split-K workspace layout for the decode entry point.
+// Most (member, head) matrix columns a wave of the cohort path carries.
+constexpr int kMaxCohortColumns = 32;
+
+// Work layout of one decode call: rows of tiles and matrix columns per pair.
+struct DecodeLayout {
+  int cols;   // columns per pair (= stride of the partial arrays)
+  int nsub;   // query sub-groups per KV head
+  int rows;   // rows of the tile sequence
+};
+inline DecodeLayout decode_layout(int n_seqs, int hn, int gn, int cohort_size) {
+  const int group = hn / gn;
+  if (cohort_size <= 1) {
+    const int gt = decode_heads_per_wave(group);
+    return {gt, (group + gt - 1) / gt, n_seqs};
+  }
+  const int cohorts = (n_seqs + cohort_size - 1) / cohort_size;
+  return {group * cohort_size, 1, cohorts * (cohort_size + 1)};
+}
+
+// Split-K workspace layout for the decode entry points.
 struct DecodeWorkspace {
-  size_t cum_bytes;  // int32 [n_seqs + 1], padded to 256
+  size_t cum_bytes;  // int32 [rows + 1], padded to 256
   size_t ml_bytes;   // float [slots, 2], padded to 256
   size_t acc_bytes;  // float [slots, hd]
   size_t total() const { return cum_bytes + ml_bytes + acc_bytes; }
 };
-inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd) {
-  const int group = hn / gn;
-  const int gt = decode_heads_per_wave(group);
-  const int nsub = (group + gt - 1) / gt;
-  // one partial per (wave, pair) segment: fewer than waves + pairs of them
-  const size_t slots = ((size_t)kMaxDecodeWaves + (size_t)n_seqs * gn * nsub) * gt;
+inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd, int cohort_size) {
+  const DecodeLayout lay = decode_layout(n_seqs, hn, gn, cohort_size);
+  // one partial per (wave, row, pair) segment: fewer than waves + rows*pairs of them
+  const size_t slots = ((size_t)kMaxDecodeWaves + (size_t)lay.rows * gn * lay.nsub) * lay.cols;
   auto pad = [](size_t n) { return (n + 255) & ~(size_t)255; };
-  return {pad(((size_t)n_seqs + 1) * sizeof(int32_t)), pad(slots * 2 * sizeof(float)),
+  return {pad(((size_t)lay.rows + 1) * sizeof(int32_t)), pad(slots * 2 * sizeof(float)),
           slots * hd * sizeof(float)};
 }
 

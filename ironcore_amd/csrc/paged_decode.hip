@@ -290,68 +290,101 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
 constexpr int kReduceThreads = 256;
 
 // Combine the split-K partials of one pair (a KV head's query heads of one
-// sequence).  grid = (pairs per sequence, n_seqs).  A pair's tiles are a
-// contiguous run of the batch-wide sequence, so the waves that touched it are
-// first_tile / chunk .. last_tile / chunk and their partial ids follow.
+// sequence).  grid = (pairs per sequence, n_seqs).  A pair's tiles in a row
+// are a contiguous run of the batch-wide sequence, so the waves that touched
+// it are first_tile / chunk .. last_tile / chunk and their partial ids follow.
+// With shared-prefix cohorts a sequence has two sources: its own row and the
+// cohort's shared row, where it owns `group` of the matrix columns.
 // Traffic is (hd+2)*4 bytes per partial, three orders of magnitude below the
 // K/V stream; what costs time here is the chain of dependent memory round
 // trips, so the prefix sums are fetched together and every thread fetches up
 // to four partials of its four output dims in one batch before it merges them
 // (a typical pair has two to four partials: two round trips in all).
-template <class E, int HD, int GT>
+template <class E, int HD>
 __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int QPH = HD / 4;  // 4-dim groups per head row
   constexpr int UB = 4;        // partials fetched per batch
   const int pair_in_seq = blockIdx.x;
   const int seq = blockIdx.y;
-  const int cum = p.cum_blocks[seq];
-  const int cum_next = p.cum_blocks[seq + 1];
-  const int cum_all = p.cum_blocks[p.n_seqs];
+  const int COLS = p.gt;
   const int kvh = pair_in_seq / p.nsub;
-  const int sub = pair_in_seq - kvh * p.nsub;
-  const int head0 = kvh * p.group + sub * GT;
-  const int heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+  int row_own = seq, row_sh = -1, col0 = 0, heads, head0;
+  if (p.cohort_size == 1) {
+    const int sub = pair_in_seq - kvh * p.nsub;
+    head0 = kvh * p.group + sub * COLS;
+    heads = (p.group - sub * COLS < COLS) ? p.group - sub * COLS : COLS;
+  } else {
+    const int co = seq / p.cohort_size;
+    const int u = seq - co * p.cohort_size;
+    row_sh = co * (p.cohort_size + 1);
+    row_own = row_sh + 1 + u;
+    col0 = u * p.group;
+    head0 = kvh * p.group;
+    heads = p.group;
+  }
+  const int cum_own = p.cum_blocks[row_own];
+  const int nb_own = p.cum_blocks[row_own + 1] - cum_own;
+  const int cum_all = p.cum_blocks[p.n_rows];
+  int cum_sh = 0, nb_sh = 0;
+  if (row_sh >= 0) {
+    cum_sh = p.cum_blocks[row_sh];
+    nb_sh = p.cum_blocks[row_sh + 1] - cum_sh;
+  }
   T *orow = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)head0 * HD;
-  const int nb = cum_next - cum;
-  if (nb == 0) {  // no visible token: zero rows
+  if (nb_own + nb_sh == 0) {  // no visible token: zero rows
     for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) orow[o] = E::narrow(0.f);
     return;
   }
   const int64_t n_tiles = (int64_t)cum_all * p.pairs_per_seq;
   const int64_t chunk = chunk_tiles(p, n_tiles);
-  const int64_t first = (int64_t)cum * p.pairs_per_seq + (int64_t)pair_in_seq * nb;
-  const int64_t w0 = first / chunk;
-  const int64_t w1 = (first + nb - 1) / chunk;
-  if (w0 == w1) return;  // one wave covered the whole pair and wrote the rows
-  const int64_t base = (int64_t)seq * p.pairs_per_seq + pair_in_seq;
+  // source 0: the shared row, source 1: the sequence's own row; an empty
+  // source gets an empty wave range
+  int64_t w_lo[2], w_hi[2], slot0[2];
+  {
+    const int64_t first = (int64_t)cum_sh * p.pairs_per_seq + (int64_t)pair_in_seq * nb_sh;
+    w_lo[0] = first / chunk;
+    w_hi[0] = nb_sh > 0 ? (first + nb_sh - 1) / chunk : w_lo[0] - 1;
+    slot0[0] = (int64_t)(row_sh < 0 ? 0 : row_sh) * p.pairs_per_seq + pair_in_seq;
+  }
+  {
+    const int64_t first = (int64_t)cum_own * p.pairs_per_seq + (int64_t)pair_in_seq * nb_own;
+    w_lo[1] = first / chunk;
+    w_hi[1] = nb_own > 0 ? (first + nb_own - 1) / chunk : w_lo[1] - 1;
+    slot0[1] = (int64_t)row_own * p.pairs_per_seq + pair_in_seq;
+  }
+  // one wave covered all the sequence has for this pair and wrote the rows
+  if (nb_sh == 0 && w_lo[1] == w_hi[1]) return;
   for (int o = threadIdx.x; o < heads * QPH; o += kReduceThreads) {
     const int g = o / QPH;
     const int d = (o - g * QPH) * 4;
     float m_run = kNegInf, l_run = 0.f;
     float4 a_run = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int64_t wb = w0; wb <= w1; wb += UB) {
-      float2 ml[UB];
-      float4 av[UB];
 #pragma unroll
-      for (int u = 0; u < UB; ++u) {  // independent loads, all in flight together
-        const int64_t w = wb + u <= w1 ? wb + u : w1;
-        const int64_t slot = (w + base) * GT + g;
-        ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
-        av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
-      }
+    for (int src = 0; src < 2; ++src) {
+      for (int64_t wb = w_lo[src]; wb <= w_hi[src]; wb += UB) {
+        float2 ml[UB];
+        float4 av[UB];
 #pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        if (wb + u > w1 || ml[u].x == kNegInf) continue;
-        const float m_new = fmaxf(m_run, ml[u].x);
-        const float keep = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
-        const float wt = __builtin_amdgcn_exp2f(ml[u].x - m_new);
-        l_run = __builtin_fmaf(ml[u].y, wt, l_run * keep);
-        a_run.x = __builtin_fmaf(av[u].x, wt, a_run.x * keep);
-        a_run.y = __builtin_fmaf(av[u].y, wt, a_run.y * keep);
-        a_run.z = __builtin_fmaf(av[u].z, wt, a_run.z * keep);
-        a_run.w = __builtin_fmaf(av[u].w, wt, a_run.w * keep);
-        m_run = m_new;
+        for (int u = 0; u < UB; ++u) {  // independent loads, all in flight together
+          const int64_t w = wb + u <= w_hi[src] ? wb + u : w_hi[src];
+          const int64_t slot = (w + slot0[src]) * COLS + col0 + g;
+          ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
+          av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
+        }
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          if (wb + u > w_hi[src] || ml[u].x == kNegInf) continue;
+          const float m_new = fmaxf(m_run, ml[u].x);
+          const float keep = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+          const float wt = __builtin_amdgcn_exp2f(ml[u].x - m_new);
+          l_run = __builtin_fmaf(ml[u].y, wt, l_run * keep);
+          a_run.x = __builtin_fmaf(av[u].x, wt, a_run.x * keep);
+          a_run.y = __builtin_fmaf(av[u].y, wt, a_run.y * keep);
+          a_run.z = __builtin_fmaf(av[u].z, wt, a_run.z * keep);
+          a_run.w = __builtin_fmaf(av[u].w, wt, a_run.w * keep);
+          m_run = m_new;
+        }
       }
     }
     const float inv = 1.f / l_run;
@@ -376,48 +409,50 @@ int resident_workgroups() {
   return per_cu * device_cu_count();
 }
 
-template <class E, int HD, int GT>
-int launch_typed(DecodeKP &kp, int dtype, hipStream_t stream) {
-  constexpr int BS = 16;
-  constexpr int NW = kDecodeWavesPerWorkgroup;
-  if constexpr (sizeof(typename E::type) == 2) {
-    // 16-bit element types: the matrix-core kernel, whatever the group size.
-    if (!launch_decode_mfma_main(kp, dtype, HD, GT, stream)) return IC_ERR_UNSUPPORTED;
-  } else {
-    int wgs = resident_workgroups<E, HD, GT, BS, NW>();
-    if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
-    kp.n_waves = wgs * NW;
-    hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
-  }
-  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD, GT>), dim3(kp.pairs_per_seq, kp.n_seqs),
+template <class E, int HD>
+int launch_reduce(const DecodeKP &kp, hipStream_t stream) {
+  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD>), dim3(kp.pairs_per_seq, kp.n_seqs),
                      dim3(kReduceThreads), 0, stream, kp);
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;
 }
 
+// fp32 pools: the vector-ALU main kernel, one instantiation per group size.
+template <class E, int HD, int GT>
+void launch_valu_main(DecodeKP &kp, hipStream_t stream) {
+  constexpr int BS = 16;
+  constexpr int NW = kDecodeWavesPerWorkgroup;
+  int wgs = resident_workgroups<E, HD, GT, BS, NW>();
+  if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
+  kp.n_waves = wgs * NW;
+  hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
+}
+
 template <class E, int HD>
-int launch_group(DecodeKP &kp, int gn, int dtype, hipStream_t stream) {
-  const int G = kp.group;
-  const int gt = decode_heads_per_wave(G);
-  kp.nsub = (G + gt - 1) / gt;
-  kp.gt = gt;
-  kp.pairs_per_seq = gn * kp.nsub;
-  switch (gt) {
-    case 1: return launch_typed<E, HD, 1>(kp, dtype, stream);
-    case 2: return launch_typed<E, HD, 2>(kp, dtype, stream);
-    case 3: return launch_typed<E, HD, 3>(kp, dtype, stream);
-    case 4: return launch_typed<E, HD, 4>(kp, dtype, stream);
-    case 5: return launch_typed<E, HD, 5>(kp, dtype, stream);
-    case 6: return launch_typed<E, HD, 6>(kp, dtype, stream);
-    case 7: return launch_typed<E, HD, 7>(kp, dtype, stream);
-    default: return launch_typed<E, HD, 8>(kp, dtype, stream);
+int launch_group(DecodeKP &kp, int dtype, hipStream_t stream) {
+  if constexpr (sizeof(typename E::type) == 2) {
+    // 16-bit element types: the matrix-core kernel, whatever the group size.
+    if (!launch_decode_mfma_main(kp, dtype, HD, stream)) return IC_ERR_UNSUPPORTED;
+  } else {
+    if (kp.cohort_size != 1) return IC_ERR_UNSUPPORTED;
+    switch (kp.gt) {
+      case 1: launch_valu_main<E, HD, 1>(kp, stream); break;
+      case 2: launch_valu_main<E, HD, 2>(kp, stream); break;
+      case 3: launch_valu_main<E, HD, 3>(kp, stream); break;
+      case 4: launch_valu_main<E, HD, 4>(kp, stream); break;
+      case 5: launch_valu_main<E, HD, 5>(kp, stream); break;
+      case 6: launch_valu_main<E, HD, 6>(kp, stream); break;
+      case 7: launch_valu_main<E, HD, 7>(kp, stream); break;
+      default: launch_valu_main<E, HD, 8>(kp, stream); break;
+    }
   }
+  return launch_reduce<E, HD>(kp, stream);
 }
 
 template <class E>
-int launch_hd(DecodeKP &kp, int hd, int gn, int dtype, hipStream_t stream) {
+int launch_hd(DecodeKP &kp, int hd, int dtype, hipStream_t stream) {
   switch (hd) {
-    case 64: return launch_group<E, 64>(kp, gn, dtype, stream);
-    case 128: return launch_group<E, 128>(kp, gn, dtype, stream);
+    case 64: return launch_group<E, 64>(kp, dtype, stream);
+    case 128: return launch_group<E, 128>(kp, dtype, stream);
     default: return IC_ERR_UNSUPPORTED;
   }
 }
@@ -448,18 +483,23 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.n_seqs = a.n_seqs;
   kp.hn = a.hn;
   kp.group = a.hn / a.gn;
-  kp.nsub = 1;
-  kp.gt = 1;
-  kp.pairs_per_seq = a.gn;
+  if (a.cohort_size > 1 && kp.group * a.cohort_size > kMaxCohortColumns) return IC_ERR_UNSUPPORTED;
+  const DecodeLayout lay = decode_layout(a.n_seqs, a.hn, a.gn, a.cohort_size);
+  kp.nsub = lay.nsub;
+  kp.gt = lay.cols;
+  kp.pairs_per_seq = a.gn * lay.nsub;
+  kp.n_rows = lay.rows;
+  kp.cohort_size = a.cohort_size > 1 ? a.cohort_size : 1;
+  kp.cohort_shared = a.cohort_size > 1 ? a.cohort_shared_blocks : nullptr;
   kp.max_ctx = a.max_context_len;
   kp.n_waves = 0;
   kp.min_chunk = (a.min_chunk_tokens + 15) / 16;
   kp.tiles_per_block = a.pool.block_size / 16;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
   switch (a.dtype) {
-    case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.gn, a.dtype, stream);
-    case IC_DTYPE_F16: return launch_hd<F16>(kp, a.hd, a.gn, a.dtype, stream);
-    case IC_DTYPE_F32: return launch_hd<F32>(kp, a.hd, a.gn, a.dtype, stream);
+    case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.dtype, stream);
+    case IC_DTYPE_F16: return launch_hd<F16>(kp, a.hd, a.dtype, stream);
+    case IC_DTYPE_F32: return launch_hd<F32>(kp, a.hd, a.dtype, stream);
     default: return IC_ERR_UNSUPPORTED;
   }
 }

@@ -98,7 +98,10 @@ __device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
   return VChunk<2>{{v.x, v.y}};
 }
 
-template <class E, int HD, int BS, int NW>
+// NCB = 16-column blocks of the query matrix a wave carries: 1 for a plain
+// pair (up to 16 heads), 2 when a shared-prefix cohort brings up to 32
+// (member, head) columns.
+template <class E, int HD, int BS, int NW, int NCB>
 __global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int ES = 2;
@@ -119,16 +122,12 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const Deco
   TileCursor c;
   if (!locate_chunk<BS>(p, lane, wid, left64, c)) return;
   // wave-uniform by construction; say so, so the bookkeeping is scalar work
-  c.seq = __builtin_amdgcn_readfirstlane(c.seq);
   c.pair = __builtin_amdgcn_readfirstlane(c.pair);
   c.blk = __builtin_amdgcn_readfirstlane(c.blk);
-  c.nb = __builtin_amdgcn_readfirstlane(c.nb);
   int left = __builtin_amdgcn_readfirstlane((int)left64);
   TileCursor walk = c;
-  TileCursor peek = c;
-  next_pair<BS>(p, peek);
   int seg_blk0 = c.blk;
-  const int GT = p.gt;
+  const int COLS = p.gt;  // columns per partial slot
 
   // K side: S row n is token (n/4) + 4(n%4).
   const int tok_k = (n >> 2) + 4 * (n & 3);
@@ -138,143 +137,207 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const Deco
 #pragma unroll
   for (int i = 0; i < NT; ++i) v_off[i] = (uint32_t)(((kg + 4 * i) * p.stride_token + n * VE) * ES);
 
-  auto pair_heads = [&](const TileCursor &tc, int &head0, int &heads) {
-    const int kvh = tc.pair / p.nsub;
-    const int sub = tc.pair - kvh * p.nsub;
-    head0 = kvh * p.group + sub * GT;
-    heads = (p.group - sub * GT < GT) ? p.group - sub * GT : GT;
+  // Matrix column col is (member col / group, head col % group) of a cohort;
+  // a lane's columns never change, so split them once: (member << 16) | head.
+  auto split = [&](int col) {
+    if (p.cohort_size == 1) return col;
+    const int u = col / p.group;
+    return (u << 16) | (col - u * p.group);
   };
-  // matrix B of q.k: head n, dims 32j + 8kg .. +7
-  auto fetch_q = [&](const TileCursor &tc, Vec16 *qq) {
-    int head0, heads;
-    pair_heads(tc, head0, heads);
+  int ug_q[NCB], ug_o[NCB][4];  // this lane's column of q.k; its four columns of the accumulators
 #pragma unroll
-    for (int j = 0; j < NK; ++j) {
-      qq[j] = Vec16{{0u, 0u, 0u, 0u}};
-      if (n < heads && tc.seq < p.n_seqs)
-        qq[j] = load16(p.q + (tc.seq * p.q_stride_seq + (int64_t)(head0 + n) * HD + 32 * j + 8 * kg) * ES);
+  for (int cb = 0; cb < NCB; ++cb) {
+    ug_q[cb] = split(cb * 16 + n);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ug_o[cb][r] = split(cb * 16 + 4 * kg + r);
+  }
+  // Wave-uniform facts about a segment's row and pair.
+  struct Segment {
+    int head0;   // first query head of the pair
+    int heads;   // query heads per member
+    int seq0;    // the row's sequence, or the cohort's first
+    int member;  // cohort rows: -1 = the shared tiles, u = member u's own tiles
+  };
+  auto segment_of = [&](const TileCursor &tc) {
+    const int kvh = tc.pair / p.nsub;
+    if (p.cohort_size == 1) {
+      const int sub = tc.pair - kvh * p.nsub;
+      const int rest = p.group - sub * COLS;
+      return Segment{kvh * p.group + sub * COLS, rest < COLS ? rest : COLS, tc.seq, -1};
+    }
+    const int rpc = p.cohort_size + 1;
+    const int co = tc.seq / rpc;
+    return Segment{kvh * p.group, p.group, co * p.cohort_size, tc.seq - co * rpc - 1};
+  };
+  Segment seg = segment_of(c);
+  // Which (sequence, query head) a matrix column of the current segment is;
+  // seq < 0 marks an unused column.
+  auto column = [&](int col, int ug, int &seq, int &head) {
+    if (p.cohort_size == 1) {
+      seq = col < seg.heads ? seg.seq0 : -1;
+      head = seg.head0 + col;
+    } else {
+      const int u = ug >> 16;
+      const int sq = seg.seq0 + u;
+      const bool on = u < p.cohort_size && sq < p.n_seqs && (seg.member < 0 || u == seg.member);
+      seq = on ? sq : -1;
+      head = seg.head0 + (ug & 0xffff);
     }
   };
-  Vec16 qreg[NK], qnext[NK];
-  fetch_q(c, qreg);
-  fetch_q(peek, qnext);
-
-  float m = kNegInf;  // reference maximum of head n (the same in all four kg groups)
-  float l = 0.f;      // sum of this lane's probabilities of head n
-  f32x4_t acc[VE];    // acc[e][r]: head 4kg + r, dim n*VE + e
+  // matrix B of q.k: column n of each block, dims 32j + 8kg .. +7
+  Vec16 qreg[NCB][NK];
+  auto fetch_q = [&]() {
 #pragma unroll
-  for (int e = 0; e < VE; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int cb = 0; cb < NCB; ++cb) {
+      int seq, head;
+      column(cb * 16 + n, ug_q[cb], seq, head);
+#pragma unroll
+      for (int j = 0; j < NK; ++j) {
+        qreg[cb][j] = Vec16{{0u, 0u, 0u, 0u}};
+        if (seq >= 0)
+          qreg[cb][j] = load16(p.q + (seq * p.q_stride_seq + (int64_t)head * HD + 32 * j + 8 * kg) * ES);
+      }
+    }
+  };
+  fetch_q();
+
+  float m[NCB], l[NCB];  // per column n: reference maximum (same in all kg groups), this lane's row sum
+  f32x4_t acc[NCB][VE];  // acc[cb][e][r]: column 16cb + 4kg + r, dim n*VE + e
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    m[cb] = kNegInf;
+    l[cb] = 0.f;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[cb][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
 
   auto finish_segment = [&]() {
-    int head0, heads;
-    pair_heads(c, head0, heads);
-    const bool whole_pair = (seg_blk0 == 0 && c.blk == c.nb);
+    // A segment that is all a sequence has (its whole row, and no shared
+    // tiles besides) writes the output rows; anything else leaves a partial.
+    const bool sole = p.cohort_size == 1 || (seg.member >= 0 && c.first == 0);
+    const bool whole_pair = sole && seg_blk0 == 0 && c.blk == c.nb;
     const int64_t partial = wid + (int64_t)c.seq * p.pairs_per_seq + c.pair;
-    float lsum = l;
-    lsum += __shfl_xor(lsum, 16, kWave);
-    lsum += __shfl_xor(lsum, 32, kWave);
-    float lr[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) lr[r] = __shfl(lsum, 4 * kg + r, kWave);
+    for (int cb = 0; cb < NCB; ++cb) {
+      float lsum = l[cb];
+      lsum += __shfl_xor(lsum, 16, kWave);
+      lsum += __shfl_xor(lsum, 32, kWave);
+      float lr[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int g = 4 * kg + r;
-      if (g < heads) {
+      for (int r = 0; r < 4; ++r) lr[r] = __shfl(lsum, 4 * kg + r, kWave);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = cb * 16 + 4 * kg + r;
+        int seq, head;
+        column(col, ug_o[cb][r], seq, head);
+        if (seq < 0) continue;
         if (whole_pair) {
           const float inv = 1.f / lr[r];
           uint32_t packed[VW];
 #pragma unroll
-          for (int k = 0; k < VW; ++k) packed[k] = E::pack(acc[2 * k][r] * inv, acc[2 * k + 1][r] * inv);
-          char *o = p.out + (c.seq * p.out_stride_seq + (int64_t)(head0 + g) * HD + n * VE) * ES;
+          for (int k = 0; k < VW; ++k)
+            packed[k] = E::pack(acc[cb][2 * k][r] * inv, acc[cb][2 * k + 1][r] * inv);
+          char *o = p.out + (seq * p.out_stride_seq + (int64_t)head * HD + n * VE) * ES;
           if (VW == 4)
             store16(o, Vec16{{packed[0], packed[1], packed[2 % VW], packed[3 % VW]}});
           else
             *reinterpret_cast<uint2 *>(o) = make_uint2(packed[0], packed[1]);
         } else {
-          float *o = p.part_acc + (partial * GT + g) * HD + n * VE;
+          float *o = p.part_acc + (partial * COLS + col) * HD + n * VE;
 #pragma unroll
           for (int k = 0; k < VE / 4; ++k)
-            *reinterpret_cast<float4 *>(o + 4 * k) =
-                make_float4(acc[4 * k][r], acc[4 * k + 1][r], acc[4 * k + 2][r], acc[4 * k + 3][r]);
+            *reinterpret_cast<float4 *>(o + 4 * k) = make_float4(acc[cb][4 * k][r], acc[cb][4 * k + 1][r],
+                                                                 acc[cb][4 * k + 2][r], acc[cb][4 * k + 3][r]);
         }
       }
-    }
-    if (!whole_pair && kg == 0 && n < heads) {
-      p.part_ml[(partial * GT + n) * 2] = m;
-      p.part_ml[(partial * GT + n) * 2 + 1] = lsum;
-    }
-    m = kNegInf;
-    l = 0.f;
+      if (!whole_pair && kg == 0) {
+        int seq, head;
+        column(cb * 16 + n, ug_q[cb], seq, head);
+        if (seq >= 0) {
+          p.part_ml[(partial * COLS + cb * 16 + n) * 2] = m[cb];
+          p.part_ml[(partial * COLS + cb * 16 + n) * 2 + 1] = lsum;
+        }
+      }
+      m[cb] = kNegInf;
+      l[cb] = 0.f;
 #pragma unroll
-    for (int e = 0; e < VE; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int e = 0; e < VE; ++e) acc[cb][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
     if (left > 0) {
-      c = peek;
+      next_pair<BS>(p, c);
       seg_blk0 = 0;
-#pragma unroll
-      for (int j = 0; j < NK; ++j) qreg[j] = qnext[j];
-      next_pair<BS>(p, peek);
-      fetch_q(peek, qnext);
+      seg = segment_of(c);
+      fetch_q();
     }
   };
 
   auto consume = [&](Vec16 *kk, VChunk<VW> *vv) {
-    // ---- scores of head n for tokens kg + 4r ------------------------------------
-    f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < NK; ++j) s4 = E::qk(kk[j], qreg[j], s4);
-    float s[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) s[r] = s4[r] * p.scale_log2e;
-    if (c.blk == c.nb - 1) {  // the sequence's last tile may be partly filled
-      int ctx = __builtin_amdgcn_readfirstlane(p.context_lens[c.seq]);
+    // The sequence's last tile may be partly filled (never a shared tile).
+    int ctx_here = 0x7fffffff;
+    const int tok0 = (c.first + c.blk) * BS;
+    if (c.blk == c.nb - 1) {
+      int ctx = __builtin_amdgcn_readfirstlane(p.context_lens[c.tseq]);
       ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
-      const int tok0 = c.blk * BS;
       if (tok0 + BS > ctx) {
+        ctx_here = ctx;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           if (tok0 + kg + 4 * r >= ctx) {
-            s[r] = kNegInf;
 #pragma unroll
             for (int k = 0; k < VW; ++k) vv[r].w[k] = 0u;
           }
         }
       }
     }
-    // ---- lazy running maximum ----------------------------------------------------
-    const float smax = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-    if (__any(smax > m + kLazyMaxSlack)) {  // rare after a segment's first tile
-      float mx = smax;
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float m_new = fmaxf(m, mx);
-      const float alpha = (m == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
-      l *= alpha;
-      m = m_new;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float ar = __shfl(alpha, 4 * kg + r, kWave);
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc[e][r] *= ar;
-      }
-    }
-    // ---- probabilities, rounded to the element type, as matrix A of p.v ----------
-    const float ms = (m == kNegInf) ? 0.f : m;
-    float pr[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      pr[r] = __builtin_amdgcn_exp2f(s[r] - ms);
-      l += pr[r];
-    }
-    const Pair32 pa = {E::pack(pr[0], pr[1]), E::pack(pr[2], pr[3])};
-    // ---- p.v: token pairs packed per dim, one MFMA per dim of this lane -----------
+    // token pairs packed per dim: matrix B of p.v, shared by all column blocks
+    Pair32 vb[VE];
 #pragma unroll
     for (int k = 0; k < VW; ++k) {
-      const Pair32 even = {__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x05040100u),
-                           __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x05040100u)};
-      const Pair32 odd = {__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x07060302u),
-                          __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x07060302u)};
-      acc[2 * k] = E::pv(pa, even, acc[2 * k]);
-      acc[2 * k + 1] = E::pv(pa, odd, acc[2 * k + 1]);
+      vb[2 * k] = Pair32{__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x05040100u),
+                         __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x05040100u)};
+      vb[2 * k + 1] = Pair32{__builtin_amdgcn_perm(vv[1].w[k], vv[0].w[k], 0x07060302u),
+                             __builtin_amdgcn_perm(vv[3].w[k], vv[2].w[k], 0x07060302u)};
+    }
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      // ---- scores of column n for tokens kg + 4r ---------------------------------
+      f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < NK; ++j) s4 = E::qk(kk[j], qreg[cb][j], s4);
+      float s[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[r] = s4[r] * p.scale_log2e;
+        if (tok0 + kg + 4 * r >= ctx_here) s[r] = kNegInf;
+      }
+      // ---- lazy running maximum --------------------------------------------------
+      const float smax = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+      if (__any(smax > m[cb] + kLazyMaxSlack)) {  // rare after a segment's first tile
+        float mx = smax;
+        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        const float m_new = fmaxf(m[cb], mx);
+        const float alpha = (m[cb] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[cb] - m_new);
+        l[cb] *= alpha;
+        m[cb] = m_new;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float ar = __shfl(alpha, 4 * kg + r, kWave);
+#pragma unroll
+          for (int e = 0; e < VE; ++e) acc[cb][e][r] *= ar;
+        }
+      }
+      // ---- probabilities, rounded to the element type, as matrix A of p.v --------
+      const float ms = (m[cb] == kNegInf) ? 0.f : m[cb];
+      float pr[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pr[r] = __builtin_amdgcn_exp2f(s[r] - ms);
+        l[cb] += pr[r];
+      }
+      const Pair32 pa = {E::pack(pr[0], pr[1]), E::pack(pr[2], pr[3])};
+#pragma unroll
+      for (int e = 0; e < VE; ++e) acc[cb][e] = E::pv(pa, vb[e], acc[cb][e]);
     }
     ++c.blk;
     --left;
@@ -317,38 +380,39 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const Deco
   }
 }
 
-template <class E, int HD>
+template <class E, int HD, int NCB>
 bool launch_one(DecodeKP &kp, hipStream_t stream) {
   constexpr int BS = 16;
   constexpr int NW = kDecodeWavesPerWorkgroup;
   static const int per_cu = [] {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_mfma_kernel<E, HD, BS, NW>, NW * kWave,
-                                                     0) != hipSuccess || n < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_mfma_kernel<E, HD, BS, NW, NCB>,
+                                                     NW * kWave, 0) != hipSuccess || n < 1)
       n = 1;
     return n;
   }();
   int wgs = per_cu * device_cu_count();
   if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
   kp.n_waves = wgs * NW;
-  hipLaunchKernelGGL((paged_decode_mfma_kernel<E, HD, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
+  hipLaunchKernelGGL((paged_decode_mfma_kernel<E, HD, BS, NW, NCB>), dim3(wgs), dim3(NW * kWave), 0, stream,
+                     kp);
   return true;
 }
 
 template <class E>
 bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
+  const bool wide = kp.gt > 16;
   switch (hd) {
-    case 64: return launch_one<E, 64>(kp, stream);
-    case 128: return launch_one<E, 128>(kp, stream);
+    case 64: return wide ? launch_one<E, 64, 2>(kp, stream) : launch_one<E, 64, 1>(kp, stream);
+    case 128: return wide ? launch_one<E, 128, 2>(kp, stream) : launch_one<E, 128, 1>(kp, stream);
     default: return false;
   }
 }
 
 }  // namespace
 
-bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, int gt, hipStream_t stream) {
-  if (gt < 1 || gt > 16) return false;
-  kp.gt = gt;
+bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream) {
+  if (kp.gt < 1 || kp.gt > 32) return false;
   switch (dtype) {
     case IC_DTYPE_BF16: return launch_hd<MfmaBf16>(kp, hd, stream);
     case IC_DTYPE_F16: return launch_hd<MfmaF16>(kp, hd, stream);

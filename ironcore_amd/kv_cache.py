@@ -153,12 +153,17 @@ class PagedKVCache:
         return blk * bs + off
 
     # ---- per-step metadata -----------------------------------------------------------
-    def prepare(self, seq_ids: Sequence[int], new_tokens: int | Iterable[int]) -> PagedAttentionMetadata:
+    def prepare(self, seq_ids: Sequence[int], new_tokens: int | Iterable[int],
+                cohort_size: int = 1) -> PagedAttentionMetadata:
         """Advance each sequence by its number of new tokens (one int for all,
         or one per sequence, padded to the longest with slot -1) and build the
         step's metadata.  The new K/V rows must then be passed through
         ``Attention.forward(..., kv_cache=cache.layer(l), attn_metadata=meta)``
-        for every layer; the same metadata serves all layers."""
+        for every layer; the same metadata serves all layers.
+
+        ``cohort_size`` > 1 groups consecutive ``seq_ids`` into cohorts and
+        records how many leading blocks each cohort's members alias (forks of
+        one prompt listed next to each other), so decode streams them once."""
         n = len(seq_ids)
         counts = [new_tokens] * n if isinstance(new_tokens, int) else list(new_tokens)
         if len(counts) != n:
@@ -177,9 +182,15 @@ class PagedKVCache:
         if any(c != width for c in counts):
             # ragged chunks: rows are padded to `width`, the kernels get true bounds
             raise NotImplementedError("per-sequence chunk lengths must be equal within one step")
+        shared = None
+        if cohort_size > 1 and n > 0:
+            from .paged_ops import shared_prefix_blocks
+            shared = torch.from_numpy(shared_prefix_blocks(table, lens, self.block_size, cohort_size)).to(dev)
         return PagedAttentionMetadata(
             block_tables=torch.tensor(table, dtype=torch.int32, device=dev).view(n, max_blocks),
             context_lens=torch.tensor(lens, dtype=torch.int32, device=dev),
             slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev),
             max_context_len=max(lens, default=0),
-            cu_seqlens_q=cu)
+            cu_seqlens_q=cu,
+            cohort_size=cohort_size if shared is not None else 1,
+            cohort_shared_blocks=shared)

@@ -43,12 +43,19 @@ class PagedAttentionMetadata:
     slot_mapping   int64 [b*sq]            pool slot of every new token, row-major
                                            over (sequence, position); -1 = padding
     max_context_len  host-side upper bound on context_lens
+    cohort_size, cohort_shared_blocks
+                   optional: consecutive groups of ``cohort_size`` sequences
+                   whose first ``cohort_shared_blocks[i]`` table entries are the
+                   same pool blocks (forked prompts); decode then reads those
+                   blocks once per cohort
     """
     block_tables: torch.Tensor
     context_lens: torch.Tensor
     slot_mapping: torch.Tensor
     max_context_len: int
     cu_seqlens_q: Optional[torch.Tensor] = None   # int32 [b+1]; built on demand for prefill
+    cohort_size: int = 1
+    cohort_shared_blocks: Optional[torch.Tensor] = None   # int32 [ceil(b / cohort_size)]
 
 
 class Attention(BaseModule):
@@ -157,8 +164,11 @@ class Attention(BaseModule):
                             meta.slot_mapping)
         scale = 1.0 / self.scale_factor
         if sq == 1:
+            cohort = meta.cohort_size if query.dtype != torch.float32 else 1
             out = paged_ops.paged_decode(query.view(b, hn, hd), k_pool, v_pool, meta.block_tables,
-                                         meta.context_lens, meta.max_context_len, scale=scale)
+                                         meta.context_lens, meta.max_context_len, scale=scale,
+                                         cohort_size=cohort,
+                                         cohort_shared_blocks=meta.cohort_shared_blocks if cohort > 1 else None)
             return out.view(b, 1, hn * hd)
         if query.dtype == torch.float32:
             return _fp32_rows_via_decode(query, k_pool, v_pool, meta.block_tables, meta.context_lens,

@@ -87,12 +87,19 @@ def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_pool: torch.Tensor, v_
 def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                  block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
                  scale: float | None = None, out: torch.Tensor | None = None,
-                 min_chunk_tokens: int = 0) -> torch.Tensor:
+                 min_chunk_tokens: int = 0, cohort_size: int = 1,
+                 cohort_shared_blocks: torch.Tensor | None = None) -> torch.Tensor:
     """One query token per sequence.  ``query`` ``[b, hn, hd]`` -> ``[b, hn*hd]``.
 
     ``max_context_len`` is a host-side upper bound on ``context_lens`` (no
     device synchronisation is needed to launch).  ``min_chunk_tokens`` is the
-    smallest split-K share (0 = library default)."""
+    smallest split-K share (0 = library default).
+
+    Shared prefixes: with ``cohort_size`` S > 1, sequences ``i*S .. i*S+S-1``
+    form cohort ``i`` and ``cohort_shared_blocks[i]`` (int32, one per cohort)
+    says how many leading block-table entries are the same pool block in all
+    of its rows; those blocks are read once per cohort.  The result is the
+    same as without cohorts."""
     lib = _lib.load()
     dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens)
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
@@ -119,16 +126,53 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
         raise ValueError("out must be [b, hn*hd] in the query dtype with contiguous rows")
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
-    need = lib.ic_paged_decode_workspace_bytes(b, hn, gn, hd)
+    cohort_size = int(cohort_size)
+    shared_ptr = 0
+    if cohort_size > 1:
+        n_cohorts = (b + cohort_size - 1) // cohort_size
+        if cohort_shared_blocks is None or cohort_shared_blocks.dtype != torch.int32 \
+                or cohort_shared_blocks.numel() != n_cohorts or not cohort_shared_blocks.is_contiguous() \
+                or cohort_shared_blocks.device != dev:
+            raise ValueError(f"cohort_shared_blocks must be a contiguous int32 [{n_cohorts}] tensor on {dev}")
+        shared_ptr = cohort_shared_blocks.data_ptr()
+    elif cohort_size < 1:
+        raise ValueError("cohort_size must be >= 1")
+    need = lib.ic_paged_decode_shared_workspace_bytes(b, hn, gn, hd, cohort_size)
+    if need == 0 and b > 0:
+        raise ValueError(f"cohort_size {cohort_size} with {hn // gn} query heads per KV head is not supported")
     ws = _workspace.get(dev, need)
     with torch.cuda.device(dev):
-        rc = lib.ic_paged_decode(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
-                                 k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
-                                 block_tables.data_ptr(), block_tables.stride(0),
-                                 context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
-                                 float(scale), min_chunk_tokens, ws.data_ptr(), ws.numel(),
-                                 _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
-    _lib.check("ic_paged_decode", rc)
+        rc = lib.ic_paged_decode_shared(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                        k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                        block_tables.data_ptr(), block_tables.stride(0),
+                                        context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
+                                        float(scale), min_chunk_tokens, cohort_size, shared_ptr,
+                                        ws.data_ptr(), ws.numel(),
+                                        _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+    _lib.check("ic_paged_decode_shared", rc)
+    return out
+
+
+def shared_prefix_blocks(block_tables, context_lens, block_size: int, cohort_size: int):
+    """Host-side helper: for each cohort of ``cohort_size`` consecutive rows of
+    ``block_tables`` (numpy or CPU tensor, ``[b, max_blocks]``), the number of
+    leading entries that are equal in all its rows and lie within every row's
+    context.  Returns an int32 numpy array ``[ceil(b / cohort_size)]``."""
+    import numpy as np
+    tables = np.asarray(block_tables)
+    ctx = np.asarray(context_lens).astype(np.int64)
+    b = tables.shape[0]
+    n_cohorts = (b + cohort_size - 1) // cohort_size
+    out = np.zeros(n_cohorts, dtype=np.int32)
+    for c in range(n_cohorts):
+        rows = tables[c * cohort_size:(c + 1) * cohort_size]
+        lim = int((ctx[c * cohort_size:(c + 1) * cohort_size] // block_size).min())
+        lim = max(min(lim, tables.shape[1]), 0)
+        if rows.shape[0] < 2 or lim == 0:
+            out[c] = lim if rows.shape[0] == 1 else 0
+            continue
+        same = (rows[1:, :lim] == rows[:1, :lim]).all(axis=0)
+        out[c] = lim if same.all() else int(np.argmin(same))
     return out
 
 

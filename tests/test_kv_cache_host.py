@@ -67,3 +67,28 @@ def test_append_into_shared_block_copies_on_write():
     new_blk = cache.blocks(c)[1]
     assert new_blk != cache.blocks(s)[1]
     assert m.slot_mapping.tolist() == [new_blk * 16 + 4]
+
+
+def test_shared_prefix_blocks_helper():
+    import numpy as np
+    from ironcore_amd.paged_ops import shared_prefix_blocks
+    tables = np.array([[7, 8, 9, 1], [7, 8, 5, 2], [3, 4, 0, 0], [3, 4, 6, 0], [9, 0, 0, 0]], dtype=np.int32)
+    ctx = np.array([64, 50, 32, 40, 10])
+    assert shared_prefix_blocks(tables, ctx, 16, 2).tolist() == [2, 2, 0]
+    assert shared_prefix_blocks(tables, ctx, 16, 4).tolist() == [0, 0]
+    # a block is only shared if every member's context covers it entirely
+    assert shared_prefix_blocks(tables, np.array([64, 20, 32, 40, 10]), 16, 2).tolist() == [1, 2, 0]
+
+
+def test_prepare_reports_cohorts_of_forked_sequences():
+    cache = PagedKVCache(1, 16, 16, 1, 4, torch.float32, "cpu")
+    s = cache.add_sequence()
+    cache.prepare([s], 40)                      # 2 full blocks + 8 tokens
+    kids = [cache.fork(s) for _ in range(3)]
+    lone = cache.add_sequence()
+    cache.prepare([lone], 5)
+    m = cache.prepare([s] + kids + [lone], 1, cohort_size=2)
+    assert m.cohort_size == 2
+    # (s, kid0) and (kid1, kid2) alias the two full prompt blocks; lone is alone in its cohort
+    assert m.cohort_shared_blocks.tolist() == [2, 2, 0]
+    assert cache.prepare([s] + kids, 1).cohort_size == 1
