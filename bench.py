@@ -35,10 +35,10 @@ import time
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
 
-# HBM bytes per launch of the decode main kernel on the default workload
-# (llama7b, seed 0), from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
-# 1 GiB device copy in the same process (profiles/paged_decode_llama7b_bs64_hbm_counters.md).
-MEASURED_TRAFFIC = {("llama7b", 0): 2466400000}
+# HBM bytes per launch of the decode main kernel (workload, seed 0), from
+# FETCH_SIZE / WRITE_SIZE counter runs scaled by a 1 GiB device copy in the
+# same process (the counter summaries under profiles/ hold the raw figures).
+MEASURED_TRAFFIC = {("llama7b", 0): 2465129779, ("llama70b", 0): 2478474342, ("grpo", 0): 997995623}
 
 
 def parse():
