@@ -11,16 +11,22 @@
 // A dense contraction, so it runs on the matrix cores
 // (v_mfma_f32_32x32x16 bf16/f16, fp32 accumulate), flash-attention style:
 //
-//  * One workgroup = a query tile of 128 rows of one query head; 4 waves, each
-//    owning a 32-row query block for the whole K/V sweep, two workgroups per
-//    CU.  The wave's Q rows stay in registers as MFMA B operands.  Workgroup
-//    ids are laid out so that all tiles and heads that read the same K/V rows
-//    run on one XCD and share its L2.
+//  * One workgroup = a query tile of 256 rows of one query head; 8 waves, each
+//    owning a 32-row query block for the whole K/V sweep (one workgroup per
+//    CU, two waves per SIMD).  The wave's Q rows stay in registers as MFMA B
+//    operands.  Workgroup ids are laid out so that all tiles and heads that
+//    read the same K/V rows run on one XCD and share its L2.
 //  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Each thread
-//    fetches its 16-byte pieces through the block table one tile ahead
-//    (table entry and base address are wave-uniform scalar work), then parks
+//    fetches its 16-byte pieces through the block table TWO tiles ahead (the
+//    table entries are scalar loads issued before the step's softmax), then parks
 //    them in double-buffered LDS, row-major ([token][dim], padded pitch).
-//    One barrier per tile.
+//    Every load is unconditional (addresses are clamped into the sequence's
+//    blocks, rows past the context are zeroed when parked), so the waits on
+//    the memory counter are exact and a tile's latency hides behind two
+//    tiles of arithmetic.
+//  * Two-sided schedule: the waves of a SIMD run half a tile apart, one in
+//    its matrix step while the other is in its vector (softmax) step, with a
+//    workgroup barrier between steps; see the loop at the end of the kernel.
 //  * Scores are computed TRANSPOSED, S^T = K Q^T: in the MFMA result layout a
 //    lane then holds one query column, so the softmax row maximum and row sum
 //    are in-lane reductions plus one exchange between the two lane halves,
@@ -75,6 +81,21 @@ struct PrefillKP {
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
+
+// x of this lane and x of lane ^ 32, as a pair (v_permlane32_swap: a vector-ALU
+// exchange, where a shuffle would be an LDS operation and share its counter).
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void both_halves(float x, float &a, float &b) {
+  const unsigned int u = __builtin_bit_cast(unsigned int, x);
+  const u32x2_t r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  unsigned int r0 = r[0], r1 = r[1];
+  // Opaque to the optimiser, which otherwise takes the two results of the swap
+  // for the same value and folds max(r0, r1) to r0.
+  asm("" : "+v"(r0), "+v"(r1));
+  a = __builtin_bit_cast(float, r0);
+  b = __builtin_bit_cast(float, r1);
+}
+
 constexpr float kLazySlack = 8.0f;  // log2 units
 
 // MFMA wrappers per element type: operands are 8 packed 16-bit values.
@@ -101,24 +122,17 @@ struct MmaF16 {
   }
 };
 
-#ifndef IC_PREFILL_QB
-#define IC_PREFILL_QB 1
-#endif
-
-constexpr int kPrefillThreads = 256;
+constexpr int kPrefillWaves = 8;
+constexpr int kPrefillThreads = kPrefillWaves * kWave;
 constexpr int kXcds = 8;
-constexpr int kBN = 64;  // tokens per K/V tile
+constexpr int kBN = 64;                   // tokens per K/V tile
+constexpr int kBM = kPrefillWaves * 32;   // query rows per workgroup
 
-// QB = 32-row query blocks per wave: a workgroup covers 4*32*QB query rows.
-// With QB = 2 every K / V^T operand read from LDS feeds two MFMAs, which
-// halves the LDS traffic per flop, and the softmax of one block overlaps the
-// matrix work of the other.
 // SINGLE: every sequence is one pool block (a dense [b, sk, gn, hd] tensor
 // viewed as a pool); otherwise blocks are a power of two >= 16 tokens long.
-template <class M, int HD, int QB, bool SINGLE>
+template <class M, int HD, bool SINGLE>
 __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const PrefillKP p) {
   using T = typename M::T;
-  constexpr int BM = 4 * 32 * QB;      // query rows per workgroup
   constexpr int KS = HD / 16;          // k-steps of the QK contraction
   constexpr int OB = HD / 32;          // 32-wide blocks of the output head dim
   constexpr int TB = kBN / 32;         // 32-token blocks per tile
@@ -146,7 +160,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int seq = unit / p.gn;
   const int kvh = unit - seq * p.gn;
   const int h = kvh * p.group + r / p.n_qtiles;
-  const int q0 = (r % p.n_qtiles) * BM;
+  const int q0 = (r % p.n_qtiles) * kBM;
   const int q_lo = p.cu_seqlens_q[seq];
   int L = p.context_lens[seq];
   int C = p.cu_seqlens_q[seq + 1] - q_lo;
@@ -157,84 +171,95 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int n = lane & 31;   // query column of this lane within a 32-row block
-  const int hh = lane >> 5;  // which half of each k-step this lane feeds
+  const int side = wave >> 2;  // 0: waves 0-3, 1: waves 4-7 (one of each per SIMD)
+  const int n = lane & 31;     // query column of this lane within the wave's 32-row block
+  const int hh = lane >> 5;    // which half of each k-step this lane feeds
 
   // ---- query rows: registers for the whole sweep, as MFMA B operands ------------
-  int limit[QB];      // last key each query row may see
-  int my_q[QB];
-  Vec16 qf[QB][KS];
+  const int my_q = q0 + wave * 32 + n;
+  const int qrow = my_q < C ? my_q : C - 1;
+  const int limit = p.causal ? P + qrow : L - 1;  // last key this query row may see
+  Vec16 qf[KS];
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    my_q[qb] = q0 + (wave * QB + qb) * 32 + n;
-    const int row = my_q[qb] < C ? my_q[qb] : C - 1;
-    limit[qb] = p.causal ? P + row : L - 1;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[qb][ks] = load16(p.q + ((q_lo + row) * p.q_stride_token + (int64_t)h * HD + ks * 16 + hh * 8) * 2);
-  }
+  for (int ks = 0; ks < KS; ++ks)
+    qf[ks] = load16(p.q + ((q_lo + qrow) * p.q_stride_token + (int64_t)h * HD + ks * 16 + hh * 8) * 2);
 
-  f32x16_t o[QB][OB];
-  float m[QB], l[QB];
+  f32x16_t o[OB];
+  float m = kNegInf, l = 0.f;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m[qb] = kNegInf;
-    l[qb] = 0.f;
+  for (int ob = 0; ob < OB; ++ob)
 #pragma unroll
-    for (int ob = 0; ob < OB; ++ob)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[qb][ob][i] = 0.f;
-  }
+    for (int i = 0; i < 16; ++i) o[ob][i] = 0.f;
 
-  int kv_end = p.causal ? P + q0 + BM : L;  // keys any row of this workgroup can see
+  int kv_end = p.causal ? P + q0 + kBM : L;  // keys any row of this workgroup can see
   kv_end = kv_end < L ? kv_end : L;
   const int n_tiles = (kv_end + kBN - 1) / kBN;
+  // tiles this wave's rows reach (the causal diagonal cuts the later ones off;
+  // a wave whose rows all lie past the end of the chunk has nothing to compute)
+  int my_end = p.causal ? P + q0 + wave * 32 + 32 : L;
+  my_end = my_end < kv_end ? my_end : kv_end;
+  const int my_tiles = (my_end > 0 && q0 + wave * 32 < C) ? (my_end + kBN - 1) / kBN : 0;
 
-  // ---- tile staging: global -> registers (one tile ahead) -> LDS -------------------
+  // ---- tile staging: global -> registers -> LDS -----------------------------------
   // In one pass the workgroup covers RPP consecutive token rows, a wave WR of
   // them.  Pool blocks are a power of two >= 16 rows long (or the sequence is a
   // single block), so the rows of one wave's pass lie inside one block: table
-  // entry, offset in the block and base address are wave-uniform scalar work
-  // and a thread only adds a fixed offset.
+  // entry and base address are wave-uniform scalar work and a thread only adds
+  // a fixed offset.  Nothing here is conditional: a tile index past the sweep
+  // is clamped to the last tile, a block index past the sequence to its last
+  // block (whose 16-row groups are allocated whether filled or not), and in
+  // SINGLE mode a row past the context to the last row.
   constexpr int WR = kWave / CPR;  // rows one wave stages per pass
   static_assert(WR <= 16 && 16 % WR == 0, "a wave's pass must stay inside a 16-row group");
   const int row0 = tid / CPR;
   const int cc = tid - row0 * CPR;
-  const uint32_t thr_off = (uint32_t)(((row0 - wave * WR) * p.stride_token + cc * 8) * 2);
+  const int row_in_wave = row0 - wave * WR;
+  const uint32_t thr_off = (uint32_t)((row_in_wave * p.stride_token + cc * 8) * 2);
   const int64_t head_off = (int64_t)kvh * p.stride_head;
-  Vec16 kst[NCH], vst[NCH];
-  auto fetch = [&](int tile) {
+  const int last_blk = SINGLE ? 0 : (L - 1) >> p.block_shift;
+  typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
+  const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
+  auto clamp_tile = [&](int tile) { return tile < n_tiles ? tile : n_tiles - 1; };
+  auto lookup = [&](int tile, int32_t *ent) {
+    tile = clamp_tile(tile);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int first = tile * kBN + i * RPP + wave * WR;  // this wave's first row of the pass
       int blk = SINGLE ? 0 : first >> p.block_shift;
-      const int rem = SINGLE ? first : first & (p.block_size - 1);
-      blk = blk < p.bt_stride ? blk : (int)p.bt_stride - 1;
-      int64_t phys = __builtin_amdgcn_readfirstlane(p.block_tables[seq * p.bt_stride + blk]);
+      blk = blk < last_blk ? blk : last_blk;
+      ent[i] = table_row[blk];
+    }
+  };
+  auto fetch_rows = [&](const char *pool, int tile, const int32_t *ent, Vec16 *st) {
+    tile = clamp_tile(tile);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int first = tile * kBN + i * RPP + wave * WR;
+      int64_t phys = ent[i];
       // A corrupt table entry must not become an out-of-pool address.
       phys = phys < 0 ? 0 : phys;
       phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
-      const int64_t base = (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2;
-      if (first + WR <= L) {
-        kst[i] = load16(p.k_pool + base + thr_off);
-        vst[i] = load16(p.v_pool + base + thr_off);
-      } else {  // the pass reaches past the context: those rows stay zero
-        kst[i] = Vec16{{0u, 0u, 0u, 0u}};
-        vst[i] = Vec16{{0u, 0u, 0u, 0u}};
-        if (tile * kBN + i * RPP + row0 < L) {
-          kst[i] = load16(p.k_pool + base + thr_off);
-          vst[i] = load16(p.v_pool + base + thr_off);
-        }
+      if (SINGLE) {
+        int row = first + row_in_wave;
+        row = row < L ? row : L - 1;
+        st[i] = load16(pool + (phys * p.stride_block + head_off + (int64_t)row * p.stride_token + cc * 8) * 2);
+      } else {
+        const int rem = first & (p.block_size - 1);
+        st[i] = load16(pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2 + thr_off);
       }
     }
   };
   const int park_k = row0 * KP + cc * 16;
   const int park_v = row0 * VP + cc * 16;
-  auto park = [&](int buf) {
+  auto park_rows = [&](char *buf, int at, int pitch, int tile, const Vec16 *st) {
+    if (tile >= n_tiles) return;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      store16(s_k[buf] + park_k + i * RPP * KP, kst[i]);
-      store16(s_v[buf] + park_v + i * RPP * VP, vst[i]);
+      const bool live = tile * kBN + i * RPP + row0 < L;  // rows past the context are parked as zeros
+      Vec16 v;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v.w[w] = live ? st[i].w[w] : 0u;
+      store16(buf + at + i * RPP * pitch, v);
     }
   };
 
@@ -242,89 +267,80 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int k_lane = n * KP + hh * 16;  // + tb*32*KP + ks*32
   const int v_lane = (4 * hh + (lane & 15) / 4) * VP + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
-  auto compute = [&](int tile, int buf) {
-    const char *sk = s_k[buf];
-    const char *sv = s_v[buf];
-    // A 32-row block whose every row ends before this tile starts has nothing to do.
-    bool active[QB];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
-      active[qb] = !p.causal || tile * kBN <= P + q0 + (wave * QB + qb) * 32 + 31;
-    if (!active[QB - 1]) return;  // blocks are ordered: the last one sees the most keys
+  f32x16_t s[TB];        // S^T of the tile in flight: (token, query n)
+  Vec16 pb[kBN / 16];    // its probabilities as MFMA B operands
 
-    // ---- S^T = K Q^T ------------------------------------------------------------
-    f32x16_t s[QB][TB];
+  // ---- S^T = K Q^T ----------------------------------------------------------------
+  auto scores = [&](int tile) {
+    const char *sk = s_k[tile & 1];
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
+    for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-      for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[qb][tb][i] = 0.f;
+      for (int i = 0; i < 16; ++i) s[tb][i] = 0.f;
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const Vec16 a = load16(sk + k_lane + tb * 32 * KP + ks * 32);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) s[qb][tb] = M::mma(a, qf[qb][ks], s[qb][tb]);
+        s[tb] = M::mma(a, qf[ks], s[tb]);
       }
     }
-    // s[qb][tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n of block qb)
+  };
+  // ---- softmax of the tile's scores: s -> pb, m, l (and o when the reference moves) ----
+  auto softmax = [&](int tile) {
+    // s[tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n)
     const int tok_base = tile * kBN + 4 * hh;
-    const bool need_mask = p.causal ? (tile * kBN + kBN - 1 > P + q0 + wave * QB * 32)
-                                    : (tile * kBN + kBN > L);
-    Vec16 pb[QB][kBN / 16];
+    const bool need_mask = p.causal ? (tile * kBN + kBN - 1 > P + q0 + wave * 32) : (tile * kBN + kBN > L);
     if (need_mask) {  // tiles that touch the causal diagonal (or the context end)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
-            s[qb][tb][i] = tok > limit[qb] ? kNegInf : s[qb][tb][i];
-          }
-    }
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      // Row maximum on the raw scores (the scale is positive), one exchange
-      // between the lane halves, then into log2 units.
-      float mx = kNegInf;
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[qb][tb][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * p.scale_log2e;
-      // Lazy reference maximum: it moves (and the accumulators are rescaled)
-      // only when some row's maximum rises by more than 2^kLazySlack above
-      // it.  Until then probabilities may exceed 1 (<= 2^kLazySlack), which
-      // fp32 sums and the 16-bit P operand hold without loss of accuracy.
-      if (__any(mx > m[qb] + kLazySlack)) {
-        const float m_new = fmaxf(m[qb], mx);
-        const float alpha = (m[qb] == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m[qb] - m_new);
-        m[qb] = m_new;
-        l[qb] *= alpha;
-#pragma unroll
-        for (int ob = 0; ob < OB; ++ob)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[qb][ob][i] *= alpha;
-      }
-      const float neg_ms = (m[qb] == kNegInf) ? 0.f : -m[qb];
-      float ps = 0.f;
-#pragma unroll
-      for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][tb][i], p.scale_log2e, neg_ms));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][tb][i + 1], p.scale_log2e, neg_ms));
-          ps += p0 + p1;
-          pb[qb][2 * tb + i / 8].w[(i & 7) / 2] = M::pack2(p0, p1);
+        for (int i = 0; i < 16; ++i) {
+          const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
+          s[tb][i] = tok > limit ? kNegInf : s[tb][i];
         }
-      }
-      l[qb] += ps;
     }
-
-    // ---- O^T += V^T P^T -----------------------------------------------------------
+    // Row maximum on the raw scores (the scale is positive), one exchange
+    // between the lane halves, then into log2 units.
+    float mx = kNegInf;
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[tb][i]);
+    float mx_a, mx_b;
+    both_halves(mx, mx_a, mx_b);
+    mx = fmaxf(mx_a, mx_b) * p.scale_log2e;
+    // Lazy reference maximum: it moves (and the accumulators are rescaled)
+    // only when some row's maximum rises by more than 2^kLazySlack above
+    // it.  Until then probabilities may exceed 1 (<= 2^kLazySlack), which
+    // fp32 sums and the 16-bit P operand hold without loss of accuracy.
+    if (__any(mx > m + kLazySlack)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = (m == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+      m = m_new;
+      l *= alpha;
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[ob][i] *= alpha;
+    }
+    const float neg_ms = (m == kNegInf) ? 0.f : -m;
+    float ps = 0.f;
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][i], p.scale_log2e, neg_ms));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][i + 1], p.scale_log2e, neg_ms));
+        ps += p0 + p1;
+        pb[2 * tb + i / 8].w[(i & 7) / 2] = M::pack2(p0, p1);
+      }
+    }
+    l += ps;
+  };
+  // ---- O^T += V^T P^T ---------------------------------------------------------------
+  auto weighted_values = [&](int tile) {
+    const char *sv = s_v[tile & 1];
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob) {
 #pragma unroll
@@ -335,62 +351,134 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
         const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) s16x4_t *)(at + 8 * VP));
         const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        const Vec16 a = __builtin_bit_cast(Vec16, both);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) o[qb][ob] = M::mma(a, pb[qb][kk], o[qb][ob]);
+        o[ob] = M::mma(__builtin_bit_cast(Vec16, both), pb[kk], o[ob]);
       }
     }
   };
 
-  // Pipeline: LDS[t&1] holds tile t while the registers carry tile t+1.  One
-  // barrier per tile.
-  fetch(0);
-  park(0);
-  if (n_tiles > 1) fetch(1);
+  // ---- two-sided pipeline ---------------------------------------------------------------
+  // A tile costs a wave about as many matrix-core cycles (K Q^T, V^T P^T) as
+  // vector-ALU cycles (softmax).  Each SIMD holds one wave of either side, and
+  // the sides run half a tile apart: in every phase one of them is in its
+  // matrix step M(k) = { O += V(k-1) P(k-1) ; S = K(k) Q } while the other is in
+  // its vector step V(k') = { P(k') = softmax(S) }, so the two pipes of a SIMD are
+  // busy at the same time.  A workgroup barrier ends each phase.
+  //   side 0:  M(0) V(0) M(1) V(1) ... M(n) V(n)  -
+  //   side 1:   -   M(0) V(0) M(1) ... V(n-1) M(n) V(n)
+  // LDS double buffers: K(k) and V(k-1) are read in phases 2k and 2k+1, so the
+  // pair {K(k+1), V(k)} ("pair k") is parked during those same two phases into
+  // the buffers K(k-1) and V(k-2) left; every thread parks its share at the end
+  // of its own vector step (side 1: in phase 2k, side 0: in phase 2k+1).
+  // Registers: a thread carries two pairs, pair k in set k & 1; once pair k is
+  // parked its set is refilled with pair k+2.
+  Vec16 kst[2][NCH], vst[2][NCH];
+  int32_t kent[NCH], vent[NCH];  // table entries of the pair the next refill fetches
+  auto lookup_pair = [&](int pair) {
+    lookup(pair + 1, kent);
+    lookup(pair, vent);
+  };
+  auto refill = [&](int pair, Vec16 *ks_, Vec16 *vs_) {
+    fetch_rows(p.k_pool, pair + 1, kent, ks_);
+    fetch_rows(p.v_pool, pair, vent, vs_);
+  };
+  auto matrix_step = [&](int k) {
+    if (k >= 1 && k <= my_tiles) weighted_values(k - 1);
+    if (k < my_tiles) {
+      scores(k);
+    } else {  // nothing to score: leave no stale value alive across the loop
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[tb][i] = 0.f;
+    }
+  };
+  auto vector_step = [&](int j, int pair, Vec16 *ks_, Vec16 *vs_) {
+    // The scalar table loads for this step's refill go first: the softmax below
+    // has no LDS or scalar-memory operation whose wait would include them.
+    lookup_pair(pair + 2);
+    if (j >= 0 && j < my_tiles) {
+      softmax(j);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < kBN / 16; ++kk) pb[kk] = Vec16{{0u, 0u, 0u, 0u}};
+    }
+    park_rows(s_k[(pair + 1) & 1], park_k, KP, pair + 1, ks_);
+    park_rows(s_v[pair & 1], park_v, VP, pair, vs_);
+    refill(pair + 2, ks_, vs_);
+  };
+  // prologue: K(0) straight into LDS, pairs 0 and 1 into the register sets
+  lookup(0, kent);
+  fetch_rows(p.k_pool, 0, kent, kst[0]);
+  park_rows(s_k[0], park_k, KP, 0, kst[0]);
+  lookup_pair(0);
+  refill(0, kst[0], vst[0]);
+  lookup_pair(1);
+  refill(1, kst[1], vst[1]);
   __syncthreads();
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    compute(tile, tile & 1);
-    if (tile + 1 < n_tiles) park((tile + 1) & 1);
+  // Both sides pass the same number of barriers.  The loops are unrolled by two
+  // so that the register set of a pair is a compile-time choice.
+  const int n_steps = (n_tiles + 2) & ~1;  // steps k = 0 .. n_steps-1 cover M(0..n_tiles), rounded up to even
+  if (side == 0) {
+    for (int k = 0; k < n_steps; k += 2) {
+      matrix_step(k);
+      __syncthreads();
+      vector_step(k, k, kst[0], vst[0]);
+      __syncthreads();
+      matrix_step(k + 1);
+      __syncthreads();
+      vector_step(k + 1, k + 1, kst[1], vst[1]);
+      __syncthreads();
+    }
     __syncthreads();
-    if (tile + 2 < n_tiles) fetch(tile + 2);
+  } else {
+    vector_step(-1, 0, kst[0], vst[0]);
+    __syncthreads();
+    for (int k = 0; k < n_steps; k += 2) {
+      matrix_step(k);
+      __syncthreads();
+      vector_step(k, k + 1, kst[1], vst[1]);
+      __syncthreads();
+      matrix_step(k + 1);
+      __syncthreads();
+      vector_step(k + 1, k + 2, kst[0], vst[0]);
+      __syncthreads();
+    }
   }
 
   // ---- normalise and store -------------------------------------------------------
+  float l_a, l_b;
+  both_halves(l, l_a, l_b);
+  const float lt = l_a + l_b;
+  const float inv = lt > 0.f ? 1.f / lt : 0.f;
+  if (my_q < C) {
+    T *orow = reinterpret_cast<T *>(p.out) + (q_lo + my_q) * p.out_stride_token + (int64_t)h * HD;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    float lt = l[qb] + __shfl_xor(l[qb], 32, kWave);
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
-    if (my_q[qb] < C) {
-      T *orow = reinterpret_cast<T *>(p.out) + (q_lo + my_q[qb]) * p.out_stride_token + (int64_t)h * HD;
+    for (int ob = 0; ob < OB; ++ob) {
 #pragma unroll
-      for (int ob = 0; ob < OB; ++ob) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int d = ob * 32 + 4 * hh + 8 * j;
-          uint2 w;
-          w.x = M::pack2(o[qb][ob][4 * j] * inv, o[qb][ob][4 * j + 1] * inv);
-          w.y = M::pack2(o[qb][ob][4 * j + 2] * inv, o[qb][ob][4 * j + 3] * inv);
-          *reinterpret_cast<uint2 *>(orow + d) = w;
-        }
+      for (int j = 0; j < 4; ++j) {
+        const int d = ob * 32 + 4 * hh + 8 * j;
+        uint2 w;
+        w.x = M::pack2(o[ob][4 * j] * inv, o[ob][4 * j + 1] * inv);
+        w.y = M::pack2(o[ob][4 * j + 2] * inv, o[ob][4 * j + 3] * inv);
+        *reinterpret_cast<uint2 *>(orow + d) = w;
       }
     }
   }
 }
 
-template <class M, int QB, bool SINGLE>
+template <class M, bool SINGLE>
 int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
-  constexpr int BM = 4 * 32 * QB;
-  kp.n_qtiles = (a.max_chunk_len + BM - 1) / BM;
+  kp.n_qtiles = (a.max_chunk_len + kBM - 1) / kBM;
   const int64_t slices = (kp.n_units + kXcds - 1) / kXcds;
   const int64_t wgs = slices * kXcds * kp.group * kp.n_qtiles;
   if (wgs > 0x7fffffff) return IC_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)wgs);
   switch (a.hd) {
     case 64:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 64, QB, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 64, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     case 128:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 128, QB, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 128, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     default:
       return IC_ERR_UNSUPPORTED;
@@ -400,11 +488,10 @@ int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
 
 template <class M>
 int launch_mode(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
-  constexpr int QB = IC_PREFILL_QB;
   // A one-column block table means one block per sequence, of any length.
-  if (a.block_table_stride == 1) return launch_hd<M, QB, true>(kp, a, stream);
+  if (a.block_table_stride == 1) return launch_hd<M, true>(kp, a, stream);
   if (kp.block_shift < 4) return IC_ERR_UNSUPPORTED;  // power-of-two blocks of >= 16 tokens
-  return launch_hd<M, QB, false>(kp, a, stream);
+  return launch_hd<M, false>(kp, a, stream);
 }
 
 }  // namespace
