@@ -76,21 +76,27 @@ def copy_calibration(torch, dev):
     torch.cuda.synchronize()
 
 
+EVENT_EVERY = 8   # steps between event pairs: recording costs launch slots of its own
+
+
 def time_steps(torch, step, steps, warmup):
     """Run `warmup` untimed steps, then exactly `steps` timed ones bracketed by
-    synchronisations.  `step(i, ev)` enqueues step i and records the event pair
-    `ev` around its dominant call.  Returns (ms per step by wall clock, list of
-    per-call ms from the events)."""
+    synchronisations.  `step(i, ev)` enqueues step i and, when `ev` is not None,
+    records the event pair `ev` around its dominant call; every EVENT_EVERY-th
+    timed step is sampled that way (an event pair per step would add two launch
+    slots to each step of the region being timed).  Returns (ms per step by
+    wall clock, list of per-call ms from the events)."""
     for i in range(warmup):
         step(i, None)
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    ev = {i: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for i in range(0, steps, EVENT_EVERY)}
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i, ev[i])
+        step(i, ev.get(i))
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in ev]
+    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in ev.values()]
 
 
 def bench_decode(args, torch, dev):
