@@ -91,6 +91,39 @@ int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
                  int dtype, void *stream);
 
 /*
+ * KV append with rotary position embedding: in one pass, rotate the query rows
+ * in place, rotate the new key rows into their cache slots and copy the new
+ * value rows into theirs.  Takes over ironcore/models/transformer.py:95-98
+ * (query = rope(query); key = rope(key)) together with the append above.
+ * Element pairs (2i, 2i+1) are rotated by the angle of table row
+ * positions[t], with the arithmetic of
+ * ironcore/layers/positional_embedding/rotary.py:69-83 (fp32, each product and
+ * sum rounded separately, result rounded to the element type), so the result
+ * is bit-identical to that expression evaluated by torch.
+ *
+ *   q              [n_tokens, hn, hd], row stride q_stride_token; rotated IN
+ *                  PLACE; NULL = no query work
+ *   k_new, v_new   as for ic_kv_append; both NULL = rotate q only (then the
+ *                  pool arguments and slot_mapping are ignored)
+ *   positions      int32 [n_tokens]: table row of each token, clamped to
+ *                  [0, table_rows).  The reference indexes its tables by the
+ *                  BATCH index of a row (rotary.py:55-64 after the transpose at
+ *                  :55); a cached decoder passes the token's position in its
+ *                  sequence.  The choice is the caller's.
+ *   cos_table, sin_table   fp32 [table_rows, hd/2], 16-byte aligned: the
+ *                  cos_emb / sin_emb buffers of rotary.py:36-51
+ */
+int ic_rope_kv_append(void *q, int64_t q_stride_token, int hn,
+                      const void *k_new, const void *v_new, int64_t new_stride_token,
+                      void *k_pool, void *v_pool,
+                      int64_t pool_stride_block, int64_t pool_stride_head,
+                      int64_t pool_stride_token,
+                      const int64_t *slot_mapping, const int32_t *positions,
+                      const float *cos_table, const float *sin_table, int64_t table_rows,
+                      int64_t n_tokens, int gn, int hd, int block_size,
+                      int64_t num_blocks, int dtype, void *stream);
+
+/*
  * Workspace the decode entry point needs (block-count prefix sums and
  * split-K partials), in bytes, for a batch of n_seqs sequences with these
  * head counts.  Returns 0 for invalid arguments.

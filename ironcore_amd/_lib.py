@@ -28,6 +28,15 @@ SIGNATURES = {
         c_void_p, c_int64,                      # slot_mapping, n_tokens
         c_int, c_int, c_int, c_int64,           # gn, hd, block_size, num_blocks
         c_int, c_void_p]),                      # dtype, stream
+    "ic_rope_kv_append": (c_int, [
+        c_void_p, c_int64, c_int,               # q, q_stride_token, hn
+        c_void_p, c_void_p, c_int64,            # k_new, v_new, new_stride_token
+        c_void_p, c_void_p,                     # k_pool, v_pool
+        c_int64, c_int64, c_int64,              # pool strides
+        c_void_p, c_void_p,                     # slot_mapping, positions
+        c_void_p, c_void_p, c_int64,            # cos_table, sin_table, table_rows
+        c_int64, c_int, c_int, c_int,           # n_tokens, gn, hd, block_size
+        c_int64, c_int, c_void_p]),             # num_blocks, dtype, stream
     "ic_paged_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "ic_paged_decode": (c_int, [
         c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride

@@ -95,6 +95,61 @@ int ic_kv_append(const void *k_new, const void *v_new, int64_t new_stride_token,
   return ic::launch_kv_append(a, static_cast<hipStream_t>(stream));
 }
 
+int ic_rope_kv_append(void *q, int64_t q_stride_token, int hn, const void *k_new, const void *v_new,
+                      int64_t new_stride_token, void *k_pool, void *v_pool, int64_t pool_stride_block,
+                      int64_t pool_stride_head, int64_t pool_stride_token, const int64_t *slot_mapping,
+                      const int32_t *positions, const float *cos_table, const float *sin_table,
+                      int64_t table_rows, int64_t n_tokens, int gn, int hd, int block_size,
+                      int64_t num_blocks, int dtype, void *stream) {
+  if (n_tokens < 0 || table_rows <= 0 || hd <= 0 || hd % 2 != 0) return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if ((hd * es) % 16 != 0) return IC_ERR_UNSUPPORTED;
+  const bool has_kv = k_new != nullptr || v_new != nullptr;
+  if (has_kv) {
+    if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                            num_blocks, es))
+      return rc;
+  }
+  if (q != nullptr && hn <= 0) return IC_ERR_BAD_SHAPE;
+  if (n_tokens == 0) return IC_OK;
+  if (!positions || !cos_table || !sin_table) return IC_ERR_NULL_POINTER;
+  if (q == nullptr && !has_kv) return IC_ERR_NULL_POINTER;
+  if (!aligned16(cos_table) || !aligned16(sin_table)) return IC_ERR_ALIGNMENT;
+  if (q != nullptr) {
+    if (q_stride_token < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
+    if (!aligned16(q) || !stride16(q_stride_token, es)) return IC_ERR_ALIGNMENT;
+  }
+  if (has_kv) {
+    if (!k_new || !v_new || !k_pool || !v_pool || !slot_mapping) return IC_ERR_NULL_POINTER;
+    if (new_stride_token < (int64_t)gn * hd) return IC_ERR_BAD_SHAPE;
+    if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_pool) || !aligned16(v_pool) ||
+        !stride16(new_stride_token, es))
+      return IC_ERR_ALIGNMENT;
+  }
+  ic::RopeAppendArgs a;
+  a.append.k_new = k_new;
+  a.append.v_new = v_new;
+  a.append.new_stride_token = new_stride_token;
+  a.append.k_pool = k_pool;
+  a.append.v_pool = v_pool;
+  a.append.pool = {pool_stride_block, pool_stride_head, pool_stride_token, has_kv ? num_blocks : 0,
+                   has_kv ? block_size : 1};
+  a.append.slot_mapping = slot_mapping;
+  a.append.n_tokens = n_tokens;
+  a.append.gn = gn;
+  a.append.hd = hd;
+  a.append.dtype = dtype;
+  a.q = q;
+  a.q_stride_token = q_stride_token;
+  a.hn = hn;
+  a.positions = positions;
+  a.cos_table = cos_table;
+  a.sin_table = sin_table;
+  a.table_rows = table_rows;
+  return ic::launch_rope_kv_append(a, static_cast<hipStream_t>(stream));
+}
+
 size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd) {
   return ic_paged_decode_shared_workspace_bytes(n_seqs, hn, gn, hd, 1);
 }

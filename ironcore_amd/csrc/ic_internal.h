@@ -30,6 +30,19 @@ struct AppendArgs {
   int dtype;
 };
 
+// KV append with rotary embedding: the plain append's arguments (k_new / v_new
+// may be null: rotate the query rows only) plus the query rows and the tables.
+struct RopeAppendArgs {
+  AppendArgs append;
+  void *q;                 // [n_tokens, hn, hd] rotated in place, or nullptr
+  int64_t q_stride_token;  // elements
+  int hn;
+  const int32_t *positions;  // [n_tokens] row of the tables each token uses
+  const float *cos_table;    // [table_rows, hd / 2]
+  const float *sin_table;
+  int64_t table_rows;
+};
+
 struct DecodeArgs {
   void *out;
   int64_t out_stride_seq;
@@ -81,6 +94,7 @@ struct PrefillArgs {
 // Each returns IC_OK, IC_ERR_UNSUPPORTED (no kernel built for this
 // dtype/shape) or IC_ERR_LAUNCH.
 int launch_kv_append(const AppendArgs &a, hipStream_t stream);
+int launch_rope_kv_append(const RopeAppendArgs &a, hipStream_t stream);
 int launch_paged_decode(const DecodeArgs &a, hipStream_t stream);
 int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream);
 

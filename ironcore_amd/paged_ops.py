@@ -84,6 +84,62 @@ def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_pool: torch.Tensor, v_
     _lib.check("ic_kv_append", rc)
 
 
+def rope_kv_append(query: torch.Tensor | None, k_new: torch.Tensor | None, v_new: torch.Tensor | None,
+                   k_pool: torch.Tensor | None, v_pool: torch.Tensor | None,
+                   slot_mapping: torch.Tensor | None, positions: torch.Tensor,
+                   cos_table: torch.Tensor, sin_table: torch.Tensor) -> None:
+    """Rotary embedding fused into the append: rotate ``query`` (``[n, hn, hd]``)
+    IN PLACE, rotate the rows of ``k_new`` into their pool slots, copy the rows
+    of ``v_new`` into theirs.  ``positions`` (int32 ``[n]``) picks each token's
+    row of the fp32 ``[rows, hd/2]`` tables.  ``query=None`` skips the query;
+    ``k_new=v_new=None`` rotates the query only."""
+    lib = _lib.load()
+    has_kv = k_new is not None
+    tensors = [positions, cos_table, sin_table]
+    tensors += [query] if query is not None else []
+    tensors += [k_new, v_new, k_pool, v_pool, slot_mapping] if has_kv else []
+    dev = _require_gpu(*tensors)
+    ref = query if query is not None else k_new
+    if ref is None:
+        raise ValueError("nothing to do: neither query nor k_new/v_new given")
+    n, hd = ref.shape[0], ref.shape[-1]
+    if cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32 or cos_table.shape != sin_table.shape \
+            or cos_table.dim() != 2 or cos_table.shape[1] != hd // 2 or not cos_table.is_contiguous() \
+            or not sin_table.is_contiguous():
+        raise ValueError(f"cos_table / sin_table must be contiguous fp32 [rows, {hd // 2}]")
+    if positions.dtype != torch.int32 or positions.numel() != n or not positions.is_contiguous():
+        raise ValueError("positions must be a contiguous int32 tensor with one entry per token")
+    q_ptr, q_stride, hn = 0, 0, 0
+    if query is not None:
+        if query.dim() != 3 or query.stride(2) != 1 or query.stride(1) != hd:
+            raise ValueError("query must be [n, hn, hd] with contiguous heads (it is rotated in place)")
+        q_ptr, q_stride, hn = query.data_ptr(), query.stride(0), query.shape[1]
+    k_ptr = v_ptr = kp_ptr = vp_ptr = slot_ptr = 0
+    new_stride = sb = sh = st = nb = 0
+    gn, bs = 1, 16
+    if has_kv:
+        nb, gn, bs, hd_pool, sb, sh, st = _pool_strides(k_pool, v_pool)
+        if hd_pool != hd or k_new.dim() != 3 or k_new.shape != v_new.shape or tuple(k_new.shape) != (n, gn, hd):
+            raise ValueError(f"k_new/v_new must be [{n}, {gn}, {hd_pool}]")
+        if not (ref.dtype == k_new.dtype == v_new.dtype == k_pool.dtype):
+            raise TypeError("query, new rows and pools must share a dtype")
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() != n or not slot_mapping.is_contiguous():
+            raise ValueError("slot_mapping must be a contiguous int64 tensor with one slot per new row")
+
+        def rows_ok(t):
+            return t.stride(2) == 1 and t.stride(1) == hd
+        if not (rows_ok(k_new) and rows_ok(v_new) and k_new.stride(0) == v_new.stride(0)):
+            k_new, v_new = k_new.contiguous(), v_new.contiguous()
+        k_ptr, v_ptr, new_stride = k_new.data_ptr(), v_new.data_ptr(), k_new.stride(0)
+        kp_ptr, vp_ptr, slot_ptr = k_pool.data_ptr(), v_pool.data_ptr(), slot_mapping.data_ptr()
+    with torch.cuda.device(dev):
+        rc = lib.ic_rope_kv_append(q_ptr, q_stride, hn, k_ptr, v_ptr, new_stride, kp_ptr, vp_ptr, sb, sh, st,
+                                   slot_ptr, positions.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(),
+                                   cos_table.shape[0], n, gn, hd, bs, nb, _lib.dtype_code(ref.dtype),
+                                   _lib.current_stream_ptr(dev))
+    _lib.check("ic_rope_kv_append", rc)
+
+
 def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                  block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
                  scale: float | None = None, out: torch.Tensor | None = None,

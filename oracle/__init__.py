@@ -13,6 +13,9 @@ paged             block-table gather + KV-append closed form that drive the
                   dense restatement through a block KV cache (the cache
                   interface is defined by this build; the reference has none).
 brute_force       independent float64 loops used to pin dense_attention.
+rope              rotary position embedding (ironcore/layers/
+                  positional_embedding/rotary.py:31-83) with the table row of a
+                  token as an explicit argument.
 gpt2              CPU restatement of the reference's GPT-2-shaped forward
                   (ironcore/language_model.py:67-100, ironcore/models/
                   transformer.py:77-132) with a full-recompute generate loop
@@ -32,6 +35,10 @@ paged.gather_kv / paged_decode /
                                   equals rows [P, P+C) of one causal pass.
 paged.kv_append                   pinned: closed form vs torch index_copy_,
                                   sentinel preservation, idempotence.
+rope.rope_tables / rope_rotate    pinned: float64 complex multiplication,
+                                  position 0 == identity, norm preservation,
+                                  relative-position property, closed-form
+                                  tables.
 gpt2.*                            pinned: cached generate == full recompute
                                   (causal-model identity); layer arithmetic vs
                                   torch.nn.functional primitives.
