@@ -256,6 +256,25 @@ def bench_prefill(args, torch, dev):
             ev[1].record()
     _, app_ms = time_steps(torch, append_only, 50, 5)
 
+    # the same append with rotary embedding fused in (Q rotated in place, K rotated
+    # into the pool, V copied), timed the same way on a scratch copy of the query
+    from oracle import rope as oracle_rope
+    cos_t, sin_t = (t.to(dev) for t in oracle_rope.rope_tables(wl.hd, 8192))
+    q_rot = wl.query.clone()
+    pos = torch.cat([torch.arange(pf, pf + c, dtype=torch.int32) for pf, c in zip(wl.prefix_lens, wl.chunk_lens)]
+                    ).to(dev)
+
+    def rope_append_only(i, ev):
+        if ev:
+            ev[0].record()
+        paged_ops.rope_kv_append(q_rot, wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping, pos,
+                                 cos_t, sin_t)
+        if ev:
+            ev[1].record()
+    _, rope_ms = time_steps(torch, rope_append_only, 50, 5)
+    rope_bytes = append_bytes + 2 * wl.query.numel() * es
+    paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)  # leave the pool unrotated
+
     result = {
         "metric": "paged_prefill_mfma_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "prefill_tokens_per_s_per_layer": round(n_tok / (ms_per_step * 1e-3), 1),
@@ -268,6 +287,7 @@ def bench_prefill(args, torch, dev):
                    "step": "kv_append(chunk rows) + paged_prefill, one layer"},
         "parity_max_abs_vs_oracle": parity,
         "append_hbm_gbps": round(append_bytes / (statistics.mean(app_ms) * 1e-3) / 1e9, 1),
+        "rope_append_hbm_gbps": round(rope_bytes / (statistics.mean(rope_ms) * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": "paged_prefill_kernel", "flops_per_launch": flops,

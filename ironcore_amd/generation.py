@@ -12,11 +12,12 @@ the full recompute by prefill + cached decode.  The GEMMs, norms and the
 activation are plain torch calls on the GPU (plumbing around the hot path);
 attention and the KV append are the HIP kernels.
 
-Only what the reference's GPT-2-shaped configuration exercises is built:
-pre/post-LN LayerNorm, learned absolute positions, GELU/ReLU/SiLU MLP, tied or
-untied output embedding.  RoPE is left out on purpose: the reference's rotary
-module indexes its angles by batch index (ironcore/layers/positional_embedding/
-rotary.py:53-64), which a KV-cached path cannot reproduce meaningfully.
+Built: pre/post-LN LayerNorm, learned absolute positions or rotary embeddings,
+GELU/ReLU/SiLU MLP, tied or untied output embedding.  Rotary embeddings use each
+token's index in its sequence; the reference's rotary module picks the angle
+of a row by its batch index (ironcore/layers/positional_embedding/
+rotary.py:53-64), which no KV-cached path can reproduce meaningfully (see
+layers/rotary.py).
 """
 from __future__ import annotations
 
@@ -30,6 +31,7 @@ from torch import nn
 from .kv_cache import PagedKVCache
 from .layers.attention import Attention
 from .layers.module import BaseModule, get_model_dtype
+from .layers.rotary import RotaryPositionalEmbedding
 
 
 class Linear(BaseModule):
@@ -106,8 +108,6 @@ class TransformerLayer(BaseModule):
 
     def forward(self, hidden_states, attention_mask, rotary_pos_emb=None, *, kv_cache=None,
                 attn_metadata=None):
-        if rotary_pos_emb is not None:
-            raise NotImplementedError("rotary embeddings are not part of the generation path")
         b, s, _ = hidden_states.shape
         norm_output = self.input_layernorm(hidden_states)
         query = self.linear_q(norm_output)
@@ -115,8 +115,16 @@ class TransformerLayer(BaseModule):
         query = query.view(b, s, self.num_local_attention_heads, self.head_dimension)
         key = key.view(b, s, self.num_local_attention_groups, self.head_dimension)
         value = value.view(b, s, self.num_local_attention_groups, self.head_dimension)
+        # transformer.py:95-98.  Without a cache the rows are rotated here, at
+        # their index in the sequence; with a cache the rotation is fused into
+        # the KV append inside the attention call.
+        if rotary_pos_emb is not None and kv_cache is None:
+            positions = torch.arange(s, device=query.device, dtype=torch.int32).repeat(b)
+            query = rotary_pos_emb(query, positions)
+            key = rotary_pos_emb(key, positions)
         attention_output = self.self_attention(query, key, value, attention_mask, kv_cache=kv_cache,
-                                               attn_metadata=attn_metadata)
+                                               attn_metadata=attn_metadata,
+                                               rotary_pos_emb=rotary_pos_emb if kv_cache is not None else None)
         attention_output = self.attn_output(attention_output)
         residual = norm_output if self.config.model.post_ln else hidden_states
         norm_input = residual + attention_output
@@ -147,13 +155,19 @@ class LanguageModelEmbedding(BaseModule):
 
     def __init__(self, config, padded_vocab_size: int):
         super().__init__(config)
-        if config.model.positional_embedding.type != "absolute":
-            raise NotImplementedError("only learned absolute positions are part of the generation path")
+        kind = config.model.positional_embedding.type
+        if kind not in ("absolute", "rope", "none"):
+            raise ValueError(f"unknown positional embedding type {kind!r}")
         self.word_embeddings = nn.Embedding(padded_vocab_size, config.model.d_model)
-        self.position_embedding = nn.Embedding(config.model.max_seq_len, config.model.d_model)
+        self.position_embedding = None
+        if kind == "absolute":  # embedding.py:16
+            self.position_embedding = nn.Embedding(config.model.max_seq_len, config.model.d_model)
 
     def forward(self, input_ids, position_ids):
-        return self.word_embeddings(input_ids) + self.position_embedding(position_ids)
+        x = self.word_embeddings(input_ids)
+        if self.position_embedding is not None:
+            x = x + self.position_embedding(position_ids)
+        return x
 
 
 def padded_vocab(vocab_size: int, unit: int = 128) -> int:
@@ -177,6 +191,12 @@ class LanguageModel(BaseModule):
         self.vocab_size = vocab_size
         self.padded_vocab_size = padded_vocab(vocab_size, config.trainer.vocab_padding_unit)
         self.embedding = LanguageModelEmbedding(config, self.padded_vocab_size)
+        self.rotary_pos_emb = None
+        if config.model.positional_embedding.type == "rope":  # language_model.py:39-47
+            pe = config.model.positional_embedding
+            self.rotary_pos_emb = RotaryPositionalEmbedding(
+                config.model.d_model // config.model.num_attention_heads, config.model.max_position_embeddings,
+                base=pe.base, scale=pe.scaling_factor, offset=pe.offset)
         self.model = TransformerModel(config)
         self.output_layernorm = LayerNorm(config)
         if config.model.untie_embed:
@@ -218,7 +238,7 @@ class LanguageModel(BaseModule):
             attention_mask = None
             position_ids = (torch.tensor(past, device=dev).unsqueeze(1) + torch.arange(s, device=dev).unsqueeze(0))
         x = self.embedding(input_ids, position_ids)
-        x = self.model(x, attention_mask, None, kv_cache=kv_cache, attn_metadata=meta)
+        x = self.model(x, attention_mask, self.rotary_pos_emb, kv_cache=kv_cache, attn_metadata=meta)
         x = self.output_layernorm(x)
         if self.config.model.untie_embed:
             return torch.matmul(x, self.output_layer.weight)

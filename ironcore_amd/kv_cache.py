@@ -169,11 +169,13 @@ class PagedKVCache:
         if len(counts) != n:
             raise ValueError("one new-token count per sequence")
         width = max(counts) if counts else 0
-        slots = []
+        slots, positions = [], []
         for sid, c in zip(seq_ids, counts):
             seq = self._seqs[sid]
+            start = seq.length
             row = [self._slot_for_append(seq) for _ in range(c)]
             slots.extend(row + [-1] * (width - c))
+            positions.extend(list(range(start, start + c)) + [0] * (width - c))
         lens = [self._seqs[s].length for s in seq_ids]
         max_blocks = max((len(self._seqs[s].blocks) for s in seq_ids), default=1) or 1
         table = [self._seqs[s].blocks + [0] * (max_blocks - len(self._seqs[s].blocks)) for s in seq_ids]
@@ -193,4 +195,5 @@ class PagedKVCache:
             max_context_len=max(lens, default=0),
             cu_seqlens_q=cu,
             cohort_size=cohort_size if shared is not None else 1,
-            cohort_shared_blocks=shared)
+            cohort_shared_blocks=shared,
+            positions=torch.tensor(positions, dtype=torch.int32, device=dev))

@@ -43,6 +43,8 @@ class PagedAttentionMetadata:
     slot_mapping   int64 [b*sq]            pool slot of every new token, row-major
                                            over (sequence, position); -1 = padding
     max_context_len  host-side upper bound on context_lens
+    positions      int32 [b*sq]            index of every new token in its sequence
+                                           (the rotary table row; 0 for padding)
     cohort_size, cohort_shared_blocks
                    optional: consecutive groups of ``cohort_size`` sequences
                    whose first ``cohort_shared_blocks[i]`` table entries are the
@@ -56,6 +58,7 @@ class PagedAttentionMetadata:
     cu_seqlens_q: Optional[torch.Tensor] = None   # int32 [b+1]; built on demand for prefill
     cohort_size: int = 1
     cohort_shared_blocks: Optional[torch.Tensor] = None   # int32 [ceil(b / cohort_size)]
+    positions: Optional[torch.Tensor] = None   # int32 [b*sq]: index of every new token in its sequence
 
 
 class Attention(BaseModule):
@@ -109,11 +112,19 @@ class Attention(BaseModule):
         raise NotImplementedError("only the causal mask (or no mask) is supported by the HIP attention path")
 
     # ------------------------------------------------------------------ forward
-    def forward(self, query, key, value, attention_mask=None, *, kv_cache=None, attn_metadata=None):
-        """query [b, sq, hn, hd]; key/value [b, sk, gn, hd]; returns [b, sq, hn*hd]."""
+    def forward(self, query, key, value, attention_mask=None, *, kv_cache=None, attn_metadata=None,
+                rotary_pos_emb=None):
+        """query [b, sq, hn, hd]; key/value [b, sk, gn, hd]; returns [b, sq, hn*hd].
+
+        ``rotary_pos_emb`` (cached path only): a rotary module whose rotation
+        of query and key has NOT been applied yet; it is fused into the KV
+        append, at the positions ``attn_metadata.positions`` names."""
         self._check_shapes(query, key, value)
         if kv_cache is not None:
-            return self._paged(query, key, value, kv_cache, attn_metadata)
+            return self._paged(query, key, value, kv_cache, attn_metadata, rotary_pos_emb)
+        if rotary_pos_emb is not None:
+            raise ValueError("without a KV cache, rotate query and key before the call "
+                             "(ironcore/models/transformer.py:95-98)")
         return self._dense(query, key, value, attention_mask)
 
     def _dense(self, query, key, value, attention_mask):
@@ -152,7 +163,7 @@ class Attention(BaseModule):
                                      torch.full((b,), sk, dtype=torch.int32, device=dev), sk, causal,
                                      1.0 / self.scale_factor)
 
-    def _paged(self, query, key, value, kv_cache, meta):
+    def _paged(self, query, key, value, kv_cache, meta, rotary_pos_emb=None):
         if meta is None:
             raise ValueError("kv_cache needs attn_metadata")
         b, sq, hn, hd = query.shape
@@ -160,8 +171,17 @@ class Attention(BaseModule):
         if key.shape[1] != sq:
             raise ValueError("with a KV cache, key/value carry only the new tokens (sk == sq)")
         k_pool, v_pool = kv_cache
-        paged_ops.kv_append(key.reshape(b * sq, gn, hd), value.reshape(b * sq, gn, hd), k_pool, v_pool,
-                            meta.slot_mapping)
+        if rotary_pos_emb is None:
+            paged_ops.kv_append(key.reshape(b * sq, gn, hd), value.reshape(b * sq, gn, hd), k_pool, v_pool,
+                                meta.slot_mapping)
+        else:
+            if meta.positions is None:
+                raise ValueError("rotary embeddings in the cached path need attn_metadata.positions")
+            rotated = query.reshape(b * sq, hn, hd).clone(memory_format=torch.contiguous_format)
+            paged_ops.rope_kv_append(rotated, key.reshape(b * sq, gn, hd), value.reshape(b * sq, gn, hd),
+                                     k_pool, v_pool, meta.slot_mapping, meta.positions,
+                                     rotary_pos_emb.cos_emb, rotary_pos_emb.sin_emb)
+            query = rotated.view(b, sq, hn, hd)
         scale = 1.0 / self.scale_factor
         if sq == 1:
             cohort = meta.cohort_size if query.dtype != torch.float32 else 1

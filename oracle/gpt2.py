@@ -26,10 +26,14 @@ import torch.nn.functional as F
 
 from . import paged as oracle_paged
 from .dense_attention import causal_offset_mask, dense_attention
+from .rope import rope_rotate
 
 
 class Dims:
-    def __init__(self, num_layers, num_heads, num_groups, d_model, ln_eps=1e-5, post_ln=False):
+    def __init__(self, num_layers, num_heads, num_groups, d_model, ln_eps=1e-5, post_ln=False, rope=None):
+        """``rope``: (cos_table, sin_table) when query and key rows are rotated
+        (transformer.py:95-98) at their index in the sequence, else None."""
+        self.rope = rope
         self.num_layers = num_layers
         self.num_heads = num_heads
         self.num_groups = num_groups
@@ -49,9 +53,25 @@ def _norm(x, w, name, eps):
     return F.layer_norm(x, (x.shape[-1],), w[name + ".layernorm.weight"], w.get(name + ".layernorm.bias"), eps)
 
 
-def _layer(x, w, prefix, dims, attend):
+def _embed(w, input_ids, pos):
+    x = F.embedding(input_ids, w["embedding.word_embeddings.weight"])
+    if "embedding.position_embedding.weight" in w:  # embedding.py:16: learned positions only when "absolute"
+        x = x + F.embedding(pos, w["embedding.position_embedding.weight"])
+    return x
+
+
+def _rotate(x, pos, dims):
+    """rotary.py:69-83 on rows [b, s, heads, hd] at positions [b, s]; the rows
+    keep the model dtype (what a cache of that dtype stores)."""
+    b, s, h, d = x.shape
+    out = rope_rotate(x.reshape(b * s, h, d), pos.reshape(-1), dims.rope[0], dims.rope[1])
+    return out.to(x.dtype).view(b, s, h, d)
+
+
+def _layer(x, w, prefix, dims, attend, pos=None):
     """One transformer block; `attend(q, k, v)` supplies the attention result
-    for q [b,s,hn,hd], k/v [b,s,gn,hd] (the new tokens' rows)."""
+    for q [b,s,hn,hd], k/v [b,s,gn,hd] (the new tokens' rows); with rotary
+    embeddings q and k are rotated at `pos` [b, s] first."""
     b, s, _ = x.shape
     norm_out = _norm(x, w, prefix + "input_layernorm", dims.ln_eps)
     q = _linear(norm_out, w, prefix + "linear_q")
@@ -59,6 +79,8 @@ def _layer(x, w, prefix, dims, attend):
     q = q.view(b, s, dims.num_heads, dims.head_dim)
     k = k.view(b, s, dims.num_groups, dims.head_dim)
     v = v.view(b, s, dims.num_groups, dims.head_dim)
+    if dims.rope is not None:
+        q, k = _rotate(q, pos, dims), _rotate(k, pos, dims)
     attn = _linear(attend(q, k, v), w, prefix + "attn_output")
     residual = norm_out if dims.post_ln else x
     norm_in = residual + attn
@@ -80,10 +102,9 @@ def forward_full(w, dims, input_ids):
     b, s = input_ids.shape
     mask = torch.tril(torch.ones(s, s)).view(1, 1, s, s) > 0.5
     pos = torch.arange(s).unsqueeze(0).expand(b, s)
-    x = F.embedding(input_ids, w["embedding.word_embeddings.weight"]) + \
-        F.embedding(pos, w["embedding.position_embedding.weight"])
+    x = _embed(w, input_ids, pos)
     for i in range(dims.num_layers):
-        x = _layer(x, w, f"model.layers.{i}.", dims, lambda q, k, v: dense_attention(q, k, v, mask))
+        x = _layer(x, w, f"model.layers.{i}.", dims, lambda q, k, v: dense_attention(q, k, v, mask), pos)
     return _logits(x, w, dims)
 
 
@@ -133,8 +154,7 @@ def forward_paged(w, dims, cache, new_ids):
     slots = cache.slots_for(s)
     ctx = torch.tensor([l + s for l in cache.lens], dtype=torch.int32)
     cu = torch.arange(0, (b + 1) * s, s, dtype=torch.int32)
-    x = F.embedding(new_ids, w["embedding.word_embeddings.weight"]) + \
-        F.embedding(pos, w["embedding.position_embedding.weight"])
+    x = _embed(w, new_ids, pos)
     for i in range(dims.num_layers):
         def attend(q, k, v, i=i):
             oracle_paged.kv_append(cache.k[i], cache.v[i], k.reshape(b * s, dims.num_groups, dims.head_dim),
@@ -142,7 +162,7 @@ def forward_paged(w, dims, cache, new_ids):
             out = oracle_paged.paged_prefill(q.reshape(b * s, dims.num_heads, dims.head_dim), cache.k[i],
                                              cache.v[i], cache.tables, ctx, cu)
             return out.view(b, s, -1)
-        x = _layer(x, w, f"model.layers.{i}.", dims, attend)
+        x = _layer(x, w, f"model.layers.{i}.", dims, attend, pos)
     cache.lens = [l + s for l in cache.lens]
     return _logits(x, w, dims)
 

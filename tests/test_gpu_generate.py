@@ -44,6 +44,32 @@ def test_small_fp32_generate_matches_oracle_tokens(gpu, groups):
     assert torch.equal(generation.generate_full_recompute(model, ids.to(gpu), 24).cpu(), want)
 
 
+def test_rotary_fp32_generate_matches_oracle_tokens(gpu):
+    """Rotary embeddings: the cached path fuses the rotation into the KV append
+    (keys enter the pool rotated at their index in the sequence), the dense
+    path rotates query and key before the call; both pick the oracle's tokens."""
+    from oracle import rope as oracle_rope
+    cfg = _small("fp32", 2)
+    cfg.model.positional_embedding.type = "rope"
+    torch.manual_seed(0)
+    model = generation.LanguageModel(cfg, vocab_size=1000)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    m = cfg.model
+    dims = oracle_gpt2.Dims(m.num_layers, m.num_attention_heads, m.num_attention_groups, m.d_model, m.ln_eps,
+                            rope=oracle_rope.rope_tables(m.d_model // m.num_attention_heads,
+                                                         m.max_position_embeddings))
+    ids = torch.randint(0, 1000, (3, 19), generator=torch.Generator().manual_seed(5))
+    want, margins = oracle_gpt2.generate_paged(w, dims, ids, 20, return_margins=True)
+    assert torch.equal(want, oracle_gpt2.generate_full_recompute(w, dims, ids, 20))
+    assert margins.min().item() > 1e-4
+    model = model.to(gpu)
+    got, got_margins = generation.generate(model, ids.to(gpu), 20, return_margins=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got.cpu(), want), f"min margin {margins.min().item()}"
+    assert (got_margins.cpu() - margins).abs().max().item() < 1e-3
+    assert torch.equal(generation.generate_full_recompute(model, ids.to(gpu), 20).cpu(), want)
+
+
 def test_small_bf16_generate_paged_equals_recompute_on_gpu(gpu):
     """bf16, like with like: cached decode and full recompute on the same device
     pick the same tokens wherever the top-1/top-2 margin is not a rounding tie."""

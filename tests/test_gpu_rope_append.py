@@ -142,3 +142,22 @@ def test_rotated_keys_give_relative_position_scores_through_decode(gpu):
         outs.append(out.float().cpu())
     assert (outs[0] - outs[1]).abs().max().item() < 3e-2
     assert (outs[0] - outs[2]).abs().max().item() < 3e-2
+
+
+def test_rotary_module_mirror(gpu):
+    """The module mirror: with positions it rotates each token by its own table
+    row; without, like the reference (rotary.py:55-64), by the row's BATCH index."""
+    from ironcore_amd.layers import RotaryPositionalEmbedding
+    rot = RotaryPositionalEmbedding(64, max_seq_len=128, base=10000, scale=1.0, offset=2).to(gpu)
+    cos, sin = oracle_rope.rope_tables(64, 128, 10000, 1.0, 2)
+    assert torch.equal(rot.cos_emb.cpu(), cos) and torch.equal(rot.sin_emb.cpu(), sin)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 5, 4, 64, generator=g).bfloat16()
+    pos = torch.randint(0, 128, (3, 5), generator=g)
+    got = rot(x.to(gpu), pos.to(gpu))
+    want = oracle_rope.rope_rotate(x.reshape(15, 4, 64), pos.reshape(-1), cos, sin).bfloat16().view(3, 5, 4, 64)
+    assert _same(got, want)
+    got = rot(x.to(gpu))
+    batch_index = torch.arange(3).repeat_interleave(5)
+    want = oracle_rope.rope_rotate(x.reshape(15, 4, 64), batch_index, cos, sin).bfloat16().view(3, 5, 4, 64)
+    assert _same(got, want)

@@ -130,3 +130,38 @@ def test_sampler_matches_reference_recipe():
     assert set(draws.flatten().tolist()) <= {1, 2}                         # only the top-2 survive
     p1 = torch.softmax(torch.tensor([3.0, 2.0]) / 0.7, 0)[0].item()
     assert abs((draws == 1).float().mean().item() - p1) < 0.08
+
+
+def _rope_dims(cfg):
+    from oracle import rope as oracle_rope
+    m = cfg.model
+    pe = m.positional_embedding
+    tables = oracle_rope.rope_tables(m.d_model // m.num_attention_heads, m.max_position_embeddings, pe.base,
+                                     pe.scaling_factor, pe.offset)
+    return oracle_gpt2.Dims(m.num_layers, m.num_attention_heads, m.num_attention_groups, m.d_model, m.ln_eps,
+                            rope=tables)
+
+
+def test_rotary_model_paged_forward_equals_full_forward_and_generates_alike():
+    """With rotary embeddings at the token's index in its sequence, keys rotated
+    once when they enter the cache serve every later step: cached passes equal
+    the full causal pass, and the rotation really matters (it changes the logits)."""
+    cfg = _tiny_config(layers=2, heads=4, groups=2)
+    cfg.model.positional_embedding.type = "rope"
+    _, w, _ = _model_and_weights(cfg, seed=9)
+    assert "embedding.position_embedding.weight" not in w
+    dims = _rope_dims(cfg)
+    ids = torch.randint(0, 300, (3, 30), generator=torch.Generator().manual_seed(4))
+    full = oracle_gpt2.forward_full(w, dims, ids)
+    cache = oracle_gpt2.OracleCache(dims, 3, 64, 16, torch.float32)
+    pre = oracle_gpt2.forward_paged(w, dims, cache, ids[:, :17])
+    torch.testing.assert_close(pre, full[:, :17], rtol=0, atol=2e-5)
+    for t in range(17, 30):
+        one = oracle_gpt2.forward_paged(w, dims, cache, ids[:, t:t + 1])
+        torch.testing.assert_close(one[:, 0], full[:, t], rtol=0, atol=2e-5)
+    m = cfg.model
+    plain = oracle_gpt2.Dims(m.num_layers, m.num_attention_heads, m.num_attention_groups, m.d_model, m.ln_eps)
+    assert (oracle_gpt2.forward_full(w, plain, ids) - full).abs().max().item() > 1e-2
+    gen_full, margins = oracle_gpt2.generate_full_recompute(w, dims, ids[:, :10], 16, return_margins=True)
+    assert margins.min().item() > 1e-4
+    assert torch.equal(gen_full, oracle_gpt2.generate_paged(w, dims, ids[:, :10], 16))
