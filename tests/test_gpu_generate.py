@@ -105,3 +105,34 @@ def test_gpt2_small_fp32_batch4_prompt128_decode64(gpu):
     print(f"min top-1/top-2 margin: oracle {margins.min().item():.3e}, gpu {got_margins.min().item():.3e}")
     assert got.shape == (4, 192)
     assert torch.equal(got.cpu(), want), f"greedy tokens differ (min margin {margins.min().item():.3e})"
+
+
+@pytest.mark.parametrize("positional", ["absolute", "rope"])
+def test_multiple_choice_scoring_matches_oracle(gpu, positional):
+    """HellaSwag-style scoring (hellaswag.py:63-88, 144-175): per-sequence mean
+    cross-entropy from one causal pass (the prefill kernel at prefix 0), lowest
+    loss wins.  Losses agree with the CPU oracle's to 1e-4 in fp32 and pick the
+    same endings."""
+    import torch.nn.functional as F
+    from ironcore_amd import scoring
+    from oracle import rope as oracle_rope
+    cfg = _small("fp32", 2)
+    cfg.model.positional_embedding.type = positional
+    torch.manual_seed(3)
+    model = generation.LanguageModel(cfg, vocab_size=1000)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    m = cfg.model
+    rope = oracle_rope.rope_tables(m.d_model // m.num_attention_heads, m.max_position_embeddings) \
+        if positional == "rope" else None
+    dims = oracle_gpt2.Dims(m.num_layers, m.num_attention_heads, m.num_attention_groups, m.d_model, m.ln_eps,
+                            rope=rope)
+    g = torch.Generator().manual_seed(8)
+    tokens = torch.randint(0, 1000, (12, 41), generator=g)           # 3 questions x 4 endings, padded length 41
+    tokens[::4, 30:] = 999                                            # some padding tails
+    logits = oracle_gpt2.forward_full(w, dims, tokens[:, :-1])
+    want = torch.stack([F.cross_entropy(logits[i], tokens[i, 1:]) for i in range(12)])
+    got = scoring.per_sample_losses(model.to(gpu).eval(), tokens.to(gpu))
+    assert (got - want).abs().max().item() < 1e-4
+    prompts = [i // 4 for i in range(12)]
+    labels = [1 if i % 4 == 2 else 0 for i in range(12)]
+    assert scoring.pick_endings(prompts, got.tolist(), labels) == scoring.pick_endings(prompts, want.tolist(), labels)

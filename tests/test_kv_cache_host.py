@@ -92,3 +92,12 @@ def test_prepare_reports_cohorts_of_forked_sequences():
     # (s, kid0) and (kid1, kid2) alias the two full prompt blocks; lone is alone in its cohort
     assert m.cohort_shared_blocks.tolist() == [2, 2, 0]
     assert cache.prepare([s] + kids, 1).cohort_size == 1
+
+
+def test_pick_endings_groups_by_prompt_and_takes_the_lowest_loss():
+    from ironcore_amd.scoring import pick_endings
+    prompts = ["a", "a", "a", "b", "b", "b"]
+    losses = [2.0, 1.0, 3.0, 0.5, 0.7, 0.9]
+    labels = [0, 1, 0, 0, 0, 1]
+    assert pick_endings(prompts, losses, labels) == {"metric": "accuracy", "score": 50.0}
+    assert pick_endings([], [], []) == 0.0
