@@ -102,7 +102,10 @@ __device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
 // pair (up to 16 heads), 2 when a shared-prefix cohort brings up to 32
 // (member, head) columns.
 template <class E, int HD, int BS, int NW, int NCB>
-__global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const DecodeKP p) {
+// Two waves per SIMD is the design point (two 8 KiB tiles in flight each); the
+// attribute keeps the two-block variant inside 256 registers.
+__global__ __launch_bounds__(NW *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void paged_decode_mfma_kernel(const DecodeKP p) {
   using T = typename E::type;
   constexpr int ES = 2;
   constexpr int NK = HD / 32;  // q.k MFMAs = 16-byte K loads per lane per tile
@@ -360,22 +363,18 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_mfma_kernel(const Deco
       __builtin_amdgcn_sched_barrier(0);
     };
 
+    // Every issue is unconditional (past the window's end it re-reads the last
+    // tile), so the waits on the memory counter stay exact and the loop body
+    // exists once.
     Vec16 ka[NK], kb[NK];
     VChunk<VW> va[NT], vb[NT];
-    int i = 0;
+    const int last = n_win - 1;
     issue(0, ka, va);
-    for (; i + 2 < n_win; i += 2) {
-      issue(i + 1, kb, vb);
+    for (int i = 0; i < n_win; i += 2) {
+      issue(i + 1 < last ? i + 1 : last, kb, vb);
       consume(ka, va);
-      issue(i + 2, ka, va);
-      consume(kb, vb);
-    }
-    if (i + 2 == n_win) {
-      issue(i + 1, kb, vb);
-      consume(ka, va);
-      consume(kb, vb);
-    } else {
-      consume(ka, va);
+      issue(i + 2 < last ? i + 2 : last, ka, va);
+      if (i + 1 < n_win) consume(kb, vb);
     }
   }
 }

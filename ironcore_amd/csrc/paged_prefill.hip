@@ -157,10 +157,28 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int unit = slice * kXcds + (within % kXcds);  // (sequence, KV head)
   if (unit >= p.n_units) return;
   const int r = within / kXcds;
-  const int seq = unit / p.gn;
+  // Longest first: workgroups are dispatched in id order and differ in length
+  // by the spread of context lengths (and, under the causal mask, by their
+  // query tile), so early ids take the longest sequences and the last query
+  // tiles.  Sequences are ranked by context length on the fly (up to one per
+  // lane).
+  int seq = unit / p.gn;
   const int kvh = unit - seq * p.gn;
+  const int n_seqs = p.n_units / p.gn;
+  if (n_seqs <= kWave) {
+    const int ln = threadIdx.x & (kWave - 1);
+    const int mine = ln < n_seqs ? p.context_lens[ln] : -0x7fffffff;
+    int rank = 0;
+    for (int j = 0; j < n_seqs; ++j) {
+      const int other = __builtin_amdgcn_readlane(mine, j);
+      rank += (other > mine || (other == mine && j < ln)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(rank == seq && ln < n_seqs);
+    seq = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit | (1ull << 63)));
+    seq = seq < n_seqs ? seq : n_seqs - 1;
+  }
   const int h = kvh * p.group + r / p.n_qtiles;
-  const int q0 = (r % p.n_qtiles) * kBM;
+  const int q0 = (p.n_qtiles - 1 - r % p.n_qtiles) * kBM;
   const int q_lo = p.cu_seqlens_q[seq];
   int L = p.context_lens[seq];
   int C = p.cu_seqlens_q[seq + 1] - q_lo;
