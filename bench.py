@@ -38,7 +38,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
 # HBM bytes per launch of the decode main kernel (workload, seed 0), from
 # FETCH_SIZE / WRITE_SIZE counter runs scaled by a 1 GiB device copy in the
 # same process (the counter summaries under profiles/ hold the raw figures).
-MEASURED_TRAFFIC = {("llama7b", 0): 2465129779, ("llama70b", 0): 2478474342, ("grpo", 0): 997995623}
+MEASURED_TRAFFIC = {("llama7b", 0): 2465132646, ("llama70b", 0): 2479168717, ("grpo", 0): 998051226}
 
 
 def parse():
