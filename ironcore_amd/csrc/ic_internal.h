@@ -98,7 +98,7 @@ int launch_rope_kv_append(const RopeAppendArgs &a, hipStream_t stream);
 int launch_paged_decode(const DecodeArgs &a, hipStream_t stream);
 int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream);
 
-constexpr int kDefaultMinChunkTokens = 128;
+constexpr int kDefaultMinChunkTokens = 16;  // one tile: short batches spread over all waves
 // Upper bound on the waves of one decode launch (sizes the workspace): 8 waves
 // on each of the 4 SIMDs of up to 512 CUs.
 constexpr int kMaxDecodeWaves = 16384;
