@@ -123,3 +123,18 @@ def test_decode_scaled_llama7b_slice(gpu):
     """The headline shape at reduced batch: Llama-7B heads, contexts in [512, 4096]."""
     wl = workloads.make_decode_workload(4, 32, 32, 128, 512, 4096, seed=0)
     _check(wl, _run(wl, gpu))
+
+
+@pytest.mark.parametrize("batch", [257, 700, 1100])
+def test_decode_many_short_sequences(gpu, batch):
+    """Batches of more than 256 and of more than 1024 sequences (the prologue
+    scans the per-sequence tile counts 256 rows at a time, and keeps them in
+    registers only up to 1024 rows), with empty sequences sprinkled in."""
+    wl = workloads.make_decode_workload(batch, 4, 2, 64, 1, 70, seed=batch)
+    wl.context_lens[::97] = 0
+    out = _run(wl, gpu)
+    ctx = wl.context_lens.clamp(min=1)
+    ref = oracle_paged.paged_decode(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, ctx)
+    ref[wl.context_lens <= 0] = 0
+    assert torch.isfinite(out.float()).all()
+    assert (out.float() - ref.float()).abs().max().item() <= TOL[wl.query.dtype]
