@@ -41,7 +41,9 @@ rope.rope_tables / rope_rotate    pinned: float64 complex multiplication,
                                   tables.
 gpt2.*                            pinned: cached generate == full recompute
                                   (causal-model identity); layer arithmetic vs
-                                  torch.nn.functional primitives.
+                                  torch.nn.functional primitives; logits and
+                                  greedy tokens vs transformers' GPT-2 on the
+                                  same random weights (tests/test_weights_hf.py).
 _flash_attention numerics         parity unpinned (third-party flash_attn wheel,
                                   absent here; ironcore/layers/attention.py:
                                   144-206).  Not restated.
