@@ -61,3 +61,21 @@ def test_positions_select_rows_per_token_not_per_batch_index():
     a = rope.rope_rotate(x, torch.tensor([4, 4, 4], dtype=torch.int32), cos, sin)
     b = rope.rope_rotate(x[1:2], torch.tensor([4], dtype=torch.int32), cos, sin)
     assert torch.equal(a[1:2], b)
+
+
+def test_against_transformers_gptj_rotary():
+    """A third-party implementation of the same interleaved-pair rotation:
+    transformers' GPT-J helpers (read as a library, not part of any reference)."""
+    import pytest
+    gptj = pytest.importorskip("transformers.models.gptj.modeling_gptj")
+    g = torch.Generator().manual_seed(7)
+    b, s, h, d = 2, 9, 3, 32
+    x = torch.randn(b, s, h, d, generator=g)
+    pos = torch.randint(0, 100, (b, s), generator=g)
+    table = gptj.create_sinusoidal_positions(100, d)                  # [100, d]: sin | cos
+    sincos = table[pos]                                               # [b, s, d]
+    sin, cos = torch.split(sincos, d // 2, dim=-1)
+    want = gptj.apply_rotary_pos_emb(x, sin, cos)
+    cos_t, sin_t = rope.rope_tables(d, 100)
+    got = rope.rope_rotate(x.reshape(b * s, h, d), pos.reshape(-1), cos_t, sin_t).view(b, s, h, d)
+    assert (got - want).abs().max().item() < 1e-5
