@@ -39,17 +39,19 @@ def _pool_strides(k_pool: torch.Tensor, v_pool: torch.Tensor):
 
 
 class _Workspace:
-    """Split-K scratch, grown on demand, one per device.  Kernels that use it
-    are stream-ordered, so reuse across calls on one stream is safe."""
+    """Split-K scratch, grown on demand, one per (device, stream).  Kernels
+    that use it are stream-ordered, so reuse across calls on one stream is
+    safe; calls on different streams get different buffers."""
 
     def __init__(self):
-        self._buf: dict[torch.device, torch.Tensor] = {}
+        self._buf: dict[tuple, torch.Tensor] = {}
 
     def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
-        buf = self._buf.get(device)
+        key = (device, _lib.current_stream_ptr(device))
+        buf = self._buf.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-            self._buf[device] = buf
+            self._buf[key] = buf
         return buf
 
 

@@ -138,3 +138,58 @@ def test_decode_many_short_sequences(gpu, batch):
     ref[wl.context_lens <= 0] = 0
     assert torch.isfinite(out.float()).all()
     assert (out.float() - ref.float()).abs().max().item() <= TOL[wl.query.dtype]
+
+
+def test_decode_step_in_a_captured_graph_and_on_two_streams(gpu):
+    """The entry points allocate nothing and only enqueue kernels, so a step
+    (append + decode) can be captured in a graph; every replay, interleaved
+    with eager work and synchronisations, must equal the eager result.  Two
+    streams running different batches at once must not disturb each other
+    (each stream has its own split-K scratch)."""
+    wl = workloads.make_decode_workload(9, 16, 4, 128, 300, 900, seed=31).to(gpu)
+    last = wl.context_lens.long() - 1
+    slots = wl.block_tables.long().gather(1, (last // 16).unsqueeze(1)).squeeze(1) * 16 + last % 16
+    g = torch.Generator(device=gpu).manual_seed(5)
+    k_new = torch.randn(9, 4, 128, generator=g, device=gpu).bfloat16()
+    v_new = torch.randn(9, 4, 128, generator=g, device=gpu).bfloat16()
+    out = torch.empty(9, 16 * 128, dtype=torch.bfloat16, device=gpu)
+
+    def step():
+        paged_ops.kv_append(k_new, v_new, wl.k_pool, wl.v_pool, slots)
+        paged_ops.paged_decode(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens,
+                               wl.max_context_len, out=out)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up on the capture stream: sizes its scratch
+    torch.cuda.current_stream().wait_stream(side)
+    step()
+    torch.cuda.synchronize()
+    want = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    for i in range(4):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
+        step()                                   # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    # two streams, two batches, launched back to back
+    wl2 = workloads.make_decode_workload(7, 16, 4, 128, 200, 1200, seed=32).to(gpu)
+    ref1 = paged_ops.paged_decode(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens, wl.max_context_len)
+    ref2 = paged_ops.paged_decode(wl2.query, wl2.k_pool, wl2.v_pool, wl2.block_tables, wl2.context_lens,
+                                  wl2.max_context_len)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(5):
+        with torch.cuda.stream(s1):
+            o1 = paged_ops.paged_decode(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens,
+                                        wl.max_context_len)
+        with torch.cuda.stream(s2):
+            o2 = paged_ops.paged_decode(wl2.query, wl2.k_pool, wl2.v_pool, wl2.block_tables, wl2.context_lens,
+                                        wl2.max_context_len)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, ref1) and torch.equal(o2, ref2)
