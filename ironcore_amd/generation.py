@@ -12,8 +12,9 @@ the full recompute by prefill + cached decode.  The GEMMs, norms and the
 activation are plain torch calls on the GPU (plumbing around the hot path);
 attention and the KV append are the HIP kernels.
 
-Built: pre/post-LN LayerNorm, learned absolute positions or rotary embeddings,
-GELU/ReLU/SiLU MLP, tied or untied output embedding.  Rotary embeddings use each
+Built: pre/post-LN with LayerNorm or RMSNorm, learned absolute positions or
+rotary embeddings, GELU/ReLU/SiLU and gated (GLU/SwiGLU/GeGLU/SiGLU) MLPs, tied or
+untied output embedding: the GPT-2 and the Llama family of shapes.  Rotary embeddings use each
 token's index in its sequence; the reference's rotary module picks the angle
 of a row by its batch index (ironcore/layers/positional_embedding/
 rotary.py:53-64), which no KV-cached path can reproduce meaningfully (see
@@ -61,25 +62,84 @@ class LayerNorm(BaseModule):
         return self.layernorm(x)
 
 
-def get_activation(name: str) -> nn.Module:
-    """ironcore/layers/activations/activations.py:45-60 (non-GLU variants)."""
+class RmsNorm(BaseModule):
+    """ironcore/layers/layernorm/fused_rms_norm.py:19-28: ``nn.RMSNorm`` under
+    the attribute ``layernorm``.  The reference also passes ``bias=`` to it,
+    which torch's RMSNorm does not take (it has a scale only), so that
+    constructor call fails there; here the scale alone is created."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.layernorm = nn.RMSNorm(config.model.d_model, eps=config.model.ln_eps)
+
+    def forward(self, x):
+        return self.layernorm(x)
+
+
+def get_layernorm(config) -> nn.Module:
+    """ironcore/layers/layernorm/__init__.py:18-26."""
+    kind = config.model.ln_type.lower()
+    if kind == "layernorm":
+        return LayerNorm(config)
+    if kind == "rmsnorm":
+        return RmsNorm(config)
+    raise NotImplementedError(f"{kind} is not supported")
+
+
+class GLUActivation(nn.Module):
+    """ironcore/layers/activations/activations.py:15-42.  The input is the
+    ``[feature | gate]`` concatenation the doubled up-projection produces;
+    ``swiglu`` is ``silu(feature) * gate``, so in Llama terms the first half of
+    the up-projection is ``gate_proj`` and the second ``up_proj``."""
+
+    def __init__(self, input_dim: int, variant: str = "glu"):
+        super().__init__()
+        self.variant = variant.lower()
+        if self.variant not in ("glu", "geglu", "siglu", "swiglu"):
+            raise ValueError(f"Unknown GLU variant: {self.variant}")
+        if self.variant in ("geglu", "siglu"):
+            self.linear = nn.Linear(input_dim, input_dim)
+
+    def forward(self, x):
+        feature, gate = x.chunk(2, dim=-1)
+        if self.variant == "glu":
+            return feature * torch.sigmoid(gate)
+        if self.variant == "geglu":
+            return self.linear(feature) * torch.sigmoid(gate)
+        if self.variant == "siglu":
+            return feature * torch.sigmoid(self.linear(gate))
+        return F.silu(feature) * gate
+
+
+def get_activation(name: str, input_dim: Optional[int] = None) -> nn.Module:
+    """ironcore/layers/activations/activations.py:45-60."""
     if name == "relu":
         return nn.ReLU()
     if name == "gelu":
         return nn.GELU()
     if name == "silu":
         return nn.SiLU()
-    raise NotImplementedError(f"activation {name!r} is not part of the generation path")
+    if "glu" in name:
+        if input_dim is None:
+            raise ValueError("input_dim is required for GLU activation")
+        return GLUActivation(input_dim, name)
+    raise NotImplementedError(f"activation {name!r}")
 
 
 class MLP(BaseModule):
-    """ironcore/layers/mlp.py:19-54 without dropout (inference)."""
+    """ironcore/layers/mlp.py:19-54 without dropout (inference): a gated
+    activation doubles the up-projection (mlp.py:31-33).  Note that the inner
+    ``nn.Linear`` of geglu/siglu is built ``d_model`` wide in the reference
+    (mlp.py:26-28) while it is applied to ``d_ffn``-wide halves, so those two
+    variants only run when ``d_ffn == d_model``; glu and swiglu have no such
+    layer."""
 
     def __init__(self, config):
         super().__init__(config)
         bias = not config.model.no_bias
-        self.activation = get_activation(config.model.activation_type)
-        self.up_proj = Linear(config, config.model.d_model, config.model.d_ffn, bias)
+        self.activation = get_activation(config.model.activation_type, config.model.d_model)
+        d_up = config.model.d_ffn * (2 if isinstance(self.activation, GLUActivation) else 1)
+        self.up_proj = Linear(config, config.model.d_model, d_up, bias)
         self.down_proj = Linear(config, config.model.d_ffn, config.model.d_model, bias)
 
     def forward(self, x):
@@ -101,9 +161,9 @@ class TransformerLayer(BaseModule):
         self.linear_q = Linear(config, m.d_model, m.head_dim * m.num_attention_heads, bias)
         self.linear_kv = Linear(config, m.d_model, m.head_dim * m.num_attention_groups * 2, bias)
         self.attn_output = Linear(config, m.head_dim * m.num_attention_heads, m.d_model, bias)
-        self.input_layernorm = LayerNorm(config)
+        self.input_layernorm = get_layernorm(config)
         self.self_attention = Attention(config)
-        self.post_attn_layernorm = LayerNorm(config)
+        self.post_attn_layernorm = get_layernorm(config)
         self.mlp = MLP(config)
 
     def forward(self, hidden_states, attention_mask, rotary_pos_emb=None, *, kv_cache=None,
@@ -198,7 +258,7 @@ class LanguageModel(BaseModule):
                 config.model.d_model // config.model.num_attention_heads, config.model.max_position_embeddings,
                 base=pe.base, scale=pe.scaling_factor, offset=pe.offset)
         self.model = TransformerModel(config)
-        self.output_layernorm = LayerNorm(config)
+        self.output_layernorm = get_layernorm(config)
         if config.model.untie_embed:
             self.output_layer = Linear(config, config.model.d_model, self.padded_vocab_size, bias=False)
         self.init_weights()

@@ -50,6 +50,18 @@ class RotaryPositionalEmbedding(nn.Module):
         self.register_buffer("sin_emb", torch.sin(idx_theta).contiguous(), persistent=False)
         self.register_buffer("cos_emb", torch.cos(idx_theta).contiguous(), persistent=False)
 
+    def _apply(self, fn, recurse=True):
+        """``model.to(torch.bfloat16)`` would round the tables (module buffers)
+        to 16 bits; the angles are fp32 by construction (rotary.py:31-51), so
+        a dtype change rebuilds them in fp32 on whatever device they moved to."""
+        super()._apply(fn, recurse)
+        if self.theta.dtype != torch.float32:
+            device = self.theta.device
+            self.theta = 1.0 / (self.rope_base ** (torch.arange(0, self.head_dim, 2, device=device).float()
+                                                   / self.head_dim))
+            self._update_rope_cache(self.max_seq_len_cached)
+        return self
+
     def forward(self, x: torch.Tensor, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``x`` ``[b, s, heads, head_dim]`` -> rotated copy.  ``positions``
         (``[b, s]`` or ``[b*s]``, any integer dtype): table row per token."""

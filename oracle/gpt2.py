@@ -1,5 +1,5 @@
-"""CPU restatement of the reference's GPT-2-shaped forward and of the two
-generate loops (TEST INFRASTRUCTURE, not product code).
+"""CPU restatement of the reference's decoder forward (GPT-2 and Llama
+shaped) and of the two generate loops (TEST INFRASTRUCTURE, not product code).
 
 Weights come in as a plain ``{name: tensor}`` dict using the reference's
 parameter names (``embedding.word_embeddings.weight``, ``model.layers.N.
@@ -8,8 +8,10 @@ linear_q.weight`` ..., weights stored ``[in, out]``).  The arithmetic follows
     ironcore/language_model.py:67-100,102-161,203-227   masks, positions, logits
     ironcore/layers/embedding.py:34-50                  word + learned position
     ironcore/models/transformer.py:77-132               pre-LN block
-    ironcore/layers/mlp.py:48-54                        up -> GELU -> down
+    ironcore/layers/mlp.py:48-54                        up -> activation -> down
+    ironcore/layers/activations/activations.py:26-39    glu / swiglu gating
     ironcore/layers/layernorm/fused_layer_norm.py:24-28 nn.LayerNorm
+    ironcore/layers/layernorm/fused_rms_norm.py:19-28   nn.RMSNorm (scale only)
     ironcore/parallel/tensor_parallel/layers.py:194-204,250-263   x @ W + b
     ironcore/layers/attention.py:68-142                 (via dense_attention)
 
@@ -30,10 +32,15 @@ from .rope import rope_rotate
 
 
 class Dims:
-    def __init__(self, num_layers, num_heads, num_groups, d_model, ln_eps=1e-5, post_ln=False, rope=None):
+    def __init__(self, num_layers, num_heads, num_groups, d_model, ln_eps=1e-5, post_ln=False, rope=None,
+                 ln_type="layernorm", activation="gelu"):
         """``rope``: (cos_table, sin_table) when query and key rows are rotated
-        (transformer.py:95-98) at their index in the sequence, else None."""
+        (transformer.py:95-98) at their index in the sequence, else None.
+        ``ln_type``: layernorm | rmsnorm.  ``activation``: gelu | relu | silu |
+        glu | swiglu."""
         self.rope = rope
+        self.ln_type = ln_type
+        self.activation = activation
         self.num_layers = num_layers
         self.num_heads = num_heads
         self.num_groups = num_groups
@@ -49,8 +56,27 @@ def _linear(x, w, name):
     return y + bias if bias is not None else y
 
 
-def _norm(x, w, name, eps):
+def _norm(x, w, name, eps, ln_type="layernorm"):
+    if ln_type == "rmsnorm":  # x / sqrt(mean(x^2) + eps) * scale, written out
+        xf = x.float()
+        y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+        return (y * w[name + ".layernorm.weight"].float()).to(x.dtype)
     return F.layer_norm(x, (x.shape[-1],), w[name + ".layernorm.weight"], w.get(name + ".layernorm.bias"), eps)
+
+
+def _activate(x, kind):
+    if kind == "gelu":
+        return F.gelu(x)
+    if kind == "relu":
+        return F.relu(x)
+    if kind == "silu":
+        return F.silu(x)
+    feature, gate = x.chunk(2, dim=-1)  # activations.py:28
+    if kind == "glu":
+        return feature * torch.sigmoid(gate)
+    if kind == "swiglu":
+        return F.silu(feature) * gate
+    raise NotImplementedError(kind)
 
 
 def _embed(w, input_ids, pos):
@@ -73,7 +99,7 @@ def _layer(x, w, prefix, dims, attend, pos=None):
     for q [b,s,hn,hd], k/v [b,s,gn,hd] (the new tokens' rows); with rotary
     embeddings q and k are rotated at `pos` [b, s] first."""
     b, s, _ = x.shape
-    norm_out = _norm(x, w, prefix + "input_layernorm", dims.ln_eps)
+    norm_out = _norm(x, w, prefix + "input_layernorm", dims.ln_eps, dims.ln_type)
     q = _linear(norm_out, w, prefix + "linear_q")
     k, v = torch.chunk(_linear(norm_out, w, prefix + "linear_kv"), 2, dim=-1)
     q = q.view(b, s, dims.num_heads, dims.head_dim)
@@ -84,14 +110,15 @@ def _layer(x, w, prefix, dims, attend, pos=None):
     attn = _linear(attend(q, k, v), w, prefix + "attn_output")
     residual = norm_out if dims.post_ln else x
     norm_in = residual + attn
-    norm_out = _norm(norm_in, w, prefix + "post_attn_layernorm", dims.ln_eps)
-    mlp = _linear(F.gelu(_linear(norm_out, w, prefix + "mlp.up_proj")), w, prefix + "mlp.down_proj")
+    norm_out = _norm(norm_in, w, prefix + "post_attn_layernorm", dims.ln_eps, dims.ln_type)
+    mlp = _linear(_activate(_linear(norm_out, w, prefix + "mlp.up_proj"), dims.activation), w,
+                  prefix + "mlp.down_proj")
     residual = norm_out if dims.post_ln else norm_in
     return residual + mlp
 
 
 def _logits(x, w, dims):
-    x = _norm(x, w, "output_layernorm", dims.ln_eps)
+    x = _norm(x, w, "output_layernorm", dims.ln_eps, dims.ln_type)
     if "output_layer.weight" in w:
         return torch.matmul(x, w["output_layer.weight"])
     return torch.matmul(x, w["embedding.word_embeddings.weight"].transpose(0, 1))

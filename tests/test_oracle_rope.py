@@ -79,3 +79,13 @@ def test_against_transformers_gptj_rotary():
     cos_t, sin_t = rope.rope_tables(d, 100)
     got = rope.rope_rotate(x.reshape(b * s, h, d), pos.reshape(-1), cos_t, sin_t).view(b, s, h, d)
     assert (got - want).abs().max().item() < 1e-5
+
+
+def test_module_tables_stay_fp32_through_a_dtype_change():
+    """``model.to(bfloat16)`` must not round the sin/cos tables."""
+    from ironcore_amd.layers.rotary import RotaryPositionalEmbedding
+    rope = RotaryPositionalEmbedding(64, 96, base=10000, offset=3)
+    sin, cos, theta = rope.sin_emb.clone(), rope.cos_emb.clone(), rope.theta.clone()
+    torch.nn.ModuleList([rope]).to(torch.bfloat16)
+    assert rope.sin_emb.dtype == torch.float32 and rope.theta.dtype == torch.float32
+    assert torch.equal(rope.sin_emb, sin) and torch.equal(rope.cos_emb, cos) and torch.equal(rope.theta, theta)

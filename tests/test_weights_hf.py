@@ -72,7 +72,9 @@ def test_logits_and_greedy_tokens_match_transformers(gpu):
         got = model(ids.to(gpu))[..., :500].cpu()
     assert (got - want).abs().max().item() < 2e-4
     with torch.no_grad():
-        hf_tokens = hf.generate(ids, max_new_tokens=24, do_sample=False, pad_token_id=0)
+        # an explicit mask: without one, generate() takes prompt tokens equal to pad_token_id for padding
+        hf_tokens = hf.generate(ids, attention_mask=torch.ones_like(ids), max_new_tokens=24, do_sample=False,
+                                pad_token_id=0)
     ours = generation.generate(model, ids.to(gpu), 24)
     torch.cuda.synchronize()
     assert torch.equal(ours.cpu(), hf_tokens)
@@ -96,5 +98,6 @@ def test_cpu_oracle_matches_transformers():
     got = oracle_gpt2.forward_full(w, dims, ids)[..., :500]
     assert (got - want).abs().max().item() < 2e-4
     with torch.no_grad():
-        hf_tokens = hf.generate(ids[:, :12], max_new_tokens=10, do_sample=False, pad_token_id=0)
+        hf_tokens = hf.generate(ids[:, :12], attention_mask=torch.ones_like(ids[:, :12]), max_new_tokens=10,
+                                 do_sample=False, pad_token_id=0)
     assert torch.equal(oracle_gpt2.generate_paged(w, dims, ids[:, :12], 10), hf_tokens)
