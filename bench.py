@@ -38,7 +38,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
 # HBM bytes per launch of the decode main kernel (workload, seed 0), from
 # FETCH_SIZE / WRITE_SIZE counter runs scaled by a 1 GiB device copy in the
 # same process (the counter summaries under profiles/ hold the raw figures).
-MEASURED_TRAFFIC = {("llama7b", 0): 2465132646, ("llama70b", 0): 2479168717, ("grpo", 0): 998051226}
+MEASURED_TRAFFIC = {("llama7b", 0): 2465266534, ("llama70b", 0): 2479865549, ("grpo", 0): 677594009}
 
 
 def parse():
@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--min-chunk-tokens", type=int, default=0, help="smallest split-K share (0 = library default)")
     ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo", "prefill"])
     ap.add_argument("--cohort-size", type=int, default=0,
-                    help="shared-prefix cohort size for decode (0 = 2 when the workload aliases prefixes, else 1)")
+                    help="shared-prefix cohort size for decode (0 = the samples per prompt of the workload, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
     ap.add_argument("--seed", type=int, default=0)
@@ -123,7 +123,7 @@ def bench_decode(args, torch, dev):
     # sequences that alias prefix blocks (GRPO samples of one prompt) are decoded in
     # cohorts that stream the shared blocks once; the sharing is a property of the
     # block tables, found on the host once, outside the timed region
-    cohort = args.cohort_size if args.cohort_size > 0 else (2 if wl.logical_tokens != wl.unique_tokens else 1)
+    cohort = args.cohort_size if args.cohort_size > 0 else int(wl.extra.get("n_samples", 1))
     shared = None
     if cohort > 1:
         shared = torch.from_numpy(paged_ops.shared_prefix_blocks(

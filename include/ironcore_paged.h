@@ -176,7 +176,10 @@ int ic_paged_decode(void *out, int64_t out_stride_seq,
  *   cohort_size           S >= 1: sequences i*S .. i*S+S-1 of the batch form
  *                         cohort i (the last one may be short).  1 = no
  *                         sharing, identical to ic_paged_decode.
- *                         (hn / gn) * S must not exceed 32; bf16 / fp16 only.
+ *                         bf16 / fp16 only; hn / gn <= 16, and S at most
+ *                         8 * (16 / (hn / gn)) (integer division): a wave
+ *                         carries the heads of 16 / (hn / gn) members and up
+ *                         to 8 waves of a workgroup share a cohort's tiles.
  *   cohort_shared_blocks  int32 [ceil(n_seqs / S)]: for each cohort, how many
  *                         leading block-table entries are the SAME pool block
  *                         in all its members' rows.  May under-state the

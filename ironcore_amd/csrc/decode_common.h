@@ -40,13 +40,22 @@ struct DecodeKP {
   float scale_log2e;
   // Shared-prefix cohorts (matrix-core kernel only).  cohort_size consecutive
   // sequences form a cohort whose first cohort_shared[c] pool blocks are the
-  // same physical blocks; those tiles are streamed once for the whole cohort.
-  // Work is laid out in ROWS: with cohort_size 1 a row is a sequence; otherwise
-  // cohort c owns rows c*(S+1) .. c*(S+1)+S: the shared tiles (all members'
-  // heads as matrix columns), then each member's private tiles.
-  const int32_t *cohort_shared;  // [ceil(n_seqs / cohort_size)] pool blocks, or nullptr
+  // same physical blocks.  The kernel then works in two phases, each with its
+  // own balanced split of its own tile sequence:
+  //   own phase     rows = sequences, each from its cohort's shared tiles on;
+  //                 a share belongs to one wave (as without cohorts);
+  //   shared phase  rows = cohorts, the shared tiles; a share belongs to a UNIT
+  //                 of 2^unit_shift neighbouring waves of one workgroup, which
+  //                 walk the same tiles at the same time, wave j of the unit
+  //                 with members j*spw .. j*spw+spw-1 as its matrix columns: the
+  //                 tile comes from HBM once and from the cache for the others.
+  const int32_t *cohort_shared;  // [n_cohorts] pool blocks, or nullptr
+  int32_t *cum_shared;           // [n_cohorts + 1] prefix sums of the shared phase's rows
+  int64_t shared_slot0;          // first partial slot of the shared phase
   int cohort_size;               // S >= 1
-  int n_rows;                    // n_seqs, or n_cohorts * (S + 1)
+  int n_cohorts;
+  int spw;
+  int unit_shift;
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
@@ -82,21 +91,22 @@ struct RowSpan {
 };
 
 template <int BS>
-__device__ __forceinline__ RowSpan row_span(const DecodeKP &p, int row) {
+__device__ __forceinline__ RowSpan row_span(const DecodeKP &p, int shared, int row) {
   if (p.cohort_size == 1) return RowSpan{row, 0, seq_blocks(p, row, BS)};
-  const int rpc = p.cohort_size + 1;
-  const int c = row / rpc;
-  const int j = row - c * rpc;
-  const int sh = cohort_shared_tiles(p, c);
-  if (j == 0) return RowSpan{c * p.cohort_size, 0, sh};
-  const int s = c * p.cohort_size + j - 1;
-  if (s >= p.n_seqs) return RowSpan{p.n_seqs - 1, 0, 0};
-  return RowSpan{s, sh, seq_blocks(p, s, BS) - sh};
+  if (shared) return RowSpan{row * p.cohort_size, 0, cohort_shared_tiles(p, row)};
+  const int sh = cohort_shared_tiles(p, row / p.cohort_size);
+  return RowSpan{row, sh, seq_blocks(p, row, BS) - sh};
 }
 
-// Tiles per wave: equal shares of the N tiles, never below min_chunk.
-__device__ __forceinline__ int64_t chunk_tiles(const DecodeKP &p, int64_t n_tiles) {
-  int64_t c = (n_tiles + p.n_waves - 1) / p.n_waves;
+// Rows and shares of a phase.
+__device__ __forceinline__ int phase_rows(const DecodeKP &p, int shared) { return shared ? p.n_cohorts : p.n_seqs; }
+__device__ __forceinline__ int phase_units(const DecodeKP &p, int shared) {
+  return shared ? p.n_waves >> p.unit_shift : p.n_waves;
+}
+
+// Tiles per share: equal shares of the N tiles, never below min_chunk.
+__device__ __forceinline__ int64_t chunk_tiles(const DecodeKP &p, int64_t n_tiles, int units) {
+  int64_t c = (n_tiles + units - 1) / units;
   return c < p.min_chunk ? p.min_chunk : c;
 }
 
@@ -128,19 +138,47 @@ __device__ __forceinline__ void set_row(TileCursor &c, int row, const RowSpan &r
   c.first = __builtin_amdgcn_readfirstlane(r.first);
 }
 
+// Where a phase's rows come from.  GlobalRows derives a row from the
+// caller's arrays every time it is asked (a few dependent loads, and one per
+// cohort member); PlannedRows reads the prefix sums a workgroup has laid out
+// in LDS once (build_plan below).
 template <int BS>
-__device__ __forceinline__ void next_pair(const DecodeKP &p, TileCursor &c) {
+struct GlobalRows {
+  const DecodeKP &p;
+  int shared;
+  __device__ __forceinline__ int n_rows() const { return phase_rows(p, shared); }
+  __device__ __forceinline__ RowSpan span(int row) const { return row_span<BS>(p, shared, row); }
+};
+
+struct PlannedRows {
+  const int *cum;     // LDS: [n + 1] exclusive prefix sums of the phase's row tile counts
+  const int *eff_sh;  // LDS: [n_cohorts] shared tiles per cohort (cohorts only)
+  int n;
+  int cohort_size;
+  int shared;
+  __device__ __forceinline__ int n_rows() const { return n; }
+  __device__ __forceinline__ RowSpan span(int row) const {
+    const int tiles = cum[row + 1] - cum[row];
+    if (cohort_size == 1) return RowSpan{row, 0, tiles};
+    if (shared) return RowSpan{row * cohort_size, 0, tiles};
+    return RowSpan{row, eff_sh[row / cohort_size], tiles};
+  }
+};
+
+template <class Rows>
+__device__ __forceinline__ void next_pair(const DecodeKP &p, const Rows &rows, TileCursor &c) {
   c.blk = 0;
   if (++c.pair == p.pairs_per_seq) {
     c.pair = 0;
+    const int n_rows = rows.n_rows();
     do {
       ++c.seq;
-      if (c.seq >= p.n_rows) {  // past the last tile: never dereferenced
-        c.seq = p.n_rows;
+      if (c.seq >= n_rows) {  // past the last tile: never dereferenced
+        c.seq = n_rows;
         c.nb = 0x7fffffff;
         return;
       }
-      set_row(c, c.seq, row_span<BS>(p, c.seq));
+      set_row(c, c.seq, rows.span(c.seq));
     } while (c.nb == 0);
   }
 }
@@ -156,26 +194,28 @@ __device__ __forceinline__ int xcd_major_workgroup() {
   return wg;
 }
 
-// This wave's share: [t0, t0 + left) of the batch-wide tile sequence and the
+// Share `wid` of a phase: [t0, t0 + left) of its tile sequence and the
 // cursor of its first tile.  Every wave prefix-sums the per-row tile counts
 // itself (kRowsPerLane consecutive rows per lane and step, their loads in
 // flight together): first for the total, which fixes the chunk size, then
-// again to find the row that holds its first tile.  Wave 0 also leaves the
+// again to find the row that holds its first tile.  Share 0 also leaves the
 // prefix sums in the workspace for the reduce kernel.  Returns false when the
 // wave has no tiles.
 constexpr int kRowsPerLane = 4;
 
 template <int BS>
-__device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int64_t wid, int64_t &left,
-                                             TileCursor &c) {
+__device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int shared, int64_t wid,
+                                             int64_t &left, TileCursor &c) {
   constexpr int RPS = kWave * kRowsPerLane;  // rows per step
+  const int n_rows = phase_rows(p, shared);
+  int32_t *cum_out = shared ? p.cum_shared : p.cum_blocks;
   int64_t total = 0;
-  for (int base = 0; base < p.n_rows; base += RPS) {
+  for (int base = 0; base < n_rows; base += RPS) {
     int cnt[kRowsPerLane];
 #pragma unroll
     for (int k = 0; k < kRowsPerLane; ++k) {
       const int r = base + lane * kRowsPerLane + k;
-      cnt[k] = r < p.n_rows ? row_span<BS>(p, r).tiles : 0;
+      cnt[k] = r < n_rows ? row_span<BS>(p, shared, r).tiles : 0;
     }
     int mine = 0;
 #pragma unroll
@@ -187,27 +227,27 @@ __device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int64_
       for (int k = 0; k < kRowsPerLane; ++k) {
         const int r = base + lane * kRowsPerLane + k;
         run += cnt[k];
-        if (r < p.n_rows) p.cum_blocks[r + 1] = run;
+        if (r < n_rows) cum_out[r + 1] = run;
       }
     }
     total += __builtin_amdgcn_readlane(incl, kWave - 1);
   }
-  if (wid == 0 && lane == 0) p.cum_blocks[0] = 0;
+  if (wid == 0 && lane == 0) cum_out[0] = 0;
   const int64_t n_tiles = total * p.pairs_per_seq;
-  const int64_t chunk = chunk_tiles(p, n_tiles);
+  const int64_t chunk = chunk_tiles(p, n_tiles, phase_units(p, shared));
   const int64_t t0 = wid * chunk;
   if (t0 >= n_tiles) return false;
   left = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;
 
   int64_t before = 0;  // tiles of the rows scanned so far
-  int row = p.n_rows;
+  int row = n_rows;
   int cum = 0;
-  for (int base = 0; base < p.n_rows; base += RPS) {
+  for (int base = 0; base < n_rows; base += RPS) {
     int cnt[kRowsPerLane];
 #pragma unroll
     for (int k = 0; k < kRowsPerLane; ++k) {
       const int r = base + lane * kRowsPerLane + k;
-      cnt[k] = r < p.n_rows ? row_span<BS>(p, r).tiles : 0;
+      cnt[k] = r < n_rows ? row_span<BS>(p, shared, r).tiles : 0;
     }
     int mine = 0;
 #pragma unroll
@@ -235,8 +275,129 @@ __device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int64_
     before += __builtin_amdgcn_readlane(incl, kWave - 1);
   }
   row = __builtin_amdgcn_readfirstlane(row);
-  set_row(c, row, row_span<BS>(p, row));
+  set_row(c, row, row_span<BS>(p, shared, row));
   const int64_t r = t0 - (int64_t)cum * p.pairs_per_seq;
+  c.pair = (int)(r / c.nb);
+  c.blk = (int)(r - (int64_t)c.pair * c.nb);
+  return true;
+}
+
+// ---- row bookkeeping in LDS ---------------------------------------------------
+// Every wave needs the prefix sums of the rows' tile counts to find its share.
+// Scanning the rows per wave (locate_chunk) costs a few dependent round trips
+// per 256 rows and, with cohorts, one load per member and row; a workgroup can
+// instead lay the prefix sums out in LDS once, all its threads sharing the
+// loads, and its waves then search LDS.  Layout (ints): eff_sh [C] | cum_sh
+// [C + 1] | cum_own [R + 1] | scratch [kPlanScratch].
+constexpr int kPlanScratch = 16;
+constexpr int kPlanMaxInts = 12000;  // 48 KB of LDS per workgroup at most
+
+struct PlanLds {
+  int *eff_sh;
+  int *cum_sh;
+  int *cum_own;
+  int *scratch;
+};
+
+__host__ __device__ inline size_t plan_ints(int n_seqs, int n_cohorts) {
+  return (size_t)n_cohorts + ((size_t)n_cohorts + 1) + ((size_t)n_seqs + 1) + kPlanScratch;
+}
+
+// The tile ring of the cooperative shared phase follows the plan, 16-byte aligned.
+__host__ __device__ inline size_t ring_offset_ints(int n_seqs, int n_cohorts) {
+  return (plan_ints(n_seqs, n_cohorts) + 3) & ~(size_t)3;
+}
+// LDS behind the plan: a K tile per wave for staging (16 rows of hd 16-bit
+// elements, padded by 16 bytes each) and, with `coop`, a ring of one such K
+// tile and one V tile per wave of the workgroup.
+__host__ __device__ constexpr size_t tiles_lds_bytes(int hd, int waves, bool coop) {
+  return (size_t)waves * (16 * (hd * 2 + 16)) + (coop ? (size_t)waves * (16 * (hd * 2 + 16) + 16 * hd * 2) : 0);
+}
+
+__device__ __forceinline__ PlanLds plan_carve(int *base, const DecodeKP &p) {
+  PlanLds pl;
+  pl.eff_sh = base;
+  pl.cum_sh = pl.eff_sh + p.n_cohorts;
+  pl.cum_own = pl.cum_sh + p.n_cohorts + 1;
+  pl.scratch = pl.cum_own + p.n_seqs + 1;
+  return pl;
+}
+
+// out[0 .. n] = exclusive prefix sums of f(0) .. f(n-1), by all T threads of
+// the workgroup (thread t takes a contiguous run of rows).  Ends with a barrier.
+template <int T, class F>
+__device__ __forceinline__ void block_prefix_sums(int n, F f, int *out, int *scratch) {
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int per = (n + T - 1) / T;
+  const int r0 = tid * per < n ? tid * per : n;
+  const int r1 = r0 + per < n ? r0 + per : n;
+  int sum = 0;
+  for (int r = r0; r < r1; ++r) sum += f(r);
+  const int incl = wave_inclusive_scan(sum, lane);
+  if (lane == kWave - 1) scratch[wave] = incl;
+  __syncthreads();
+  int run = incl - sum, total = 0;
+#pragma unroll
+  for (int w = 0; w < T / kWave; ++w) {
+    const int v = scratch[w];
+    run += w < wave ? v : 0;
+    total += v;
+  }
+  for (int r = r0; r < r1; ++r) {
+    out[r] = run;
+    run += f(r);
+  }
+  if (tid == 0) out[n] = total;
+  __syncthreads();
+}
+
+// Builds the plan; `publish` (one workgroup of the grid) also leaves the prefix
+// sums in the workspace for the reduce kernel.
+template <int BS, int T>
+__device__ __forceinline__ void build_plan(const DecodeKP &p, const PlanLds &pl, bool publish) {
+  const int tid = threadIdx.x;
+  const bool cohorts = p.cohort_size > 1;
+  if (cohorts) {
+    for (int c = tid; c < p.n_cohorts; c += T) pl.eff_sh[c] = cohort_shared_tiles(p, c);
+    __syncthreads();
+    block_prefix_sums<T>(p.n_cohorts, [&](int c) { return pl.eff_sh[c]; }, pl.cum_sh, pl.scratch);
+    block_prefix_sums<T>(p.n_seqs, [&](int r) { return seq_blocks(p, r, BS) - pl.eff_sh[r / p.cohort_size]; },
+                         pl.cum_own, pl.scratch);
+  } else {
+    block_prefix_sums<T>(p.n_seqs, [&](int r) { return seq_blocks(p, r, BS); }, pl.cum_own, pl.scratch);
+  }
+  if (publish) {
+    for (int r = tid; r <= p.n_seqs; r += T) p.cum_blocks[r] = pl.cum_own[r];
+    if (cohorts)
+      for (int c = tid; c <= p.n_cohorts; c += T) p.cum_shared[c] = pl.cum_sh[c];
+  }
+}
+
+// locate_chunk on a plan: share `wid` of `units` of the phase whose prefix
+// sums are cum[0 .. n_rows].  64-way search: each round the lanes probe 64
+// evenly spaced entries of the bracket.
+__device__ __forceinline__ bool locate_planned(const DecodeKP &p, const PlannedRows &rows, int units, int lane,
+                                               int64_t wid, int64_t &left, TileCursor &c) {
+  const int n_rows = rows.n;
+  const int64_t n_tiles = (int64_t)rows.cum[n_rows] * p.pairs_per_seq;
+  const int64_t chunk = chunk_tiles(p, n_tiles, units);
+  const int64_t t0 = wid * chunk;
+  if (t0 >= n_tiles) return false;
+  left = (t0 + chunk < n_tiles ? t0 + chunk : n_tiles) - t0;
+  int lo = 0, hi = n_rows;  // the row is the last one in [lo, hi) whose prefix sum does not exceed t0
+  while (hi - lo > 1) {
+    const int step = (hi - lo + kWave - 1) / kWave;
+    const int idx = lo + lane * step;
+    const int v = rows.cum[idx < hi ? idx : hi];
+    const uint64_t over = __ballot(idx >= hi || (int64_t)v * p.pairs_per_seq > t0);
+    const int f = over != 0 ? __builtin_ctzll(over) : kWave;  // lane 0 probes lo: never over
+    const int lo_new = lo + (f - 1) * step;
+    hi = lo + f * step < hi ? lo + f * step : hi;
+    lo = lo_new;
+  }
+  const int row = __builtin_amdgcn_readfirstlane(lo);
+  set_row(c, row, rows.span(row));
+  const int64_t r = t0 - (int64_t)rows.cum[row] * p.pairs_per_seq;
   c.pair = (int)(r / c.nb);
   c.blk = (int)(r - (int64_t)c.pair * c.nb);
   return true;
@@ -245,9 +406,9 @@ __device__ __forceinline__ bool locate_chunk(const DecodeKP &p, int lane, int64_
 // Window = the next n_win (<= 64*SW) tiles of the share.  Each lane looks up
 // the pool block of SW of them and keeps the tile's byte offset (the same for
 // the K and the V pool); `walk` advances past the window.
-template <int BS, int SW, int ES>
-__device__ __forceinline__ void gather_window(const DecodeKP &p, int lane, int n_win, TileCursor &walk,
-                                              uint32_t *off_lo, uint32_t *off_hi) {
+template <int BS, int SW, int ES, class Rows>
+__device__ __forceinline__ void gather_window(const DecodeKP &p, const Rows &rows, int lane, int n_win,
+                                              TileCursor &walk, uint32_t *off_lo, uint32_t *off_hi) {
   int64_t row_idx[SW];
   int32_t kv_of[SW], sub_of[SW];
 #pragma unroll
@@ -277,7 +438,7 @@ __device__ __forceinline__ void gather_window(const DecodeKP &p, int lane, int n
     }
     pos += cnt;
     walk.blk += cnt;
-    if (walk.blk == walk.nb) next_pair<BS>(p, walk);
+    if (walk.blk == walk.nb) next_pair(p, rows, walk);
   }
 #pragma unroll
   for (int r = 0; r < SW; ++r) {
@@ -316,7 +477,7 @@ __device__ __forceinline__ int64_t window_tile_offset(const uint32_t *off_lo, co
 constexpr int kDecodeWavesPerWorkgroup = 4;
 
 // Launches the matrix-core decode main kernel (paged_decode_mfma.hip) when it
-// is built for this shape (16-bit dtype, hd 64 or 128, kp.gt <= 32 columns);
+// is built for this shape (16-bit dtype, hd 64 or 128, kp.gt <= 16 columns);
 // returns false otherwise.  Sets kp.n_waves.
 bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream);
 

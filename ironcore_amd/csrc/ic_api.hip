@@ -156,7 +156,7 @@ size_t ic_paged_decode_workspace_bytes(int n_seqs, int hn, int gn, int hd) {
 
 size_t ic_paged_decode_shared_workspace_bytes(int n_seqs, int hn, int gn, int hd, int cohort_size) {
   if (n_seqs <= 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0 || cohort_size < 1) return 0;
-  if (cohort_size > 1 && (hn / gn) * cohort_size > ic::kMaxCohortColumns) return 0;
+  if (!ic::decode_layout(n_seqs, hn, gn, cohort_size).ok) return 0;
   return ic::decode_workspace(n_seqs, hn, gn, hd, cohort_size).total();
 }
 
@@ -193,7 +193,7 @@ int ic_paged_decode_shared(void *out, int64_t out_stride_seq, const void *q, int
   if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
   if (cohort_size > 1) {
     if (!cohort_shared_blocks) return IC_ERR_NULL_POINTER;
-    if (dtype == IC_DTYPE_F32 || (hn / gn) * cohort_size > ic::kMaxCohortColumns) return IC_ERR_UNSUPPORTED;
+    if (dtype == IC_DTYPE_F32 || !ic::decode_layout(n_seqs, hn, gn, cohort_size).ok) return IC_ERR_UNSUPPORTED;
   }
   if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
   if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
@@ -231,6 +231,7 @@ int ic_paged_decode_shared(void *out, int64_t out_stride_seq, const void *q, int
   a.cum_blocks = reinterpret_cast<int32_t *>(wsp);
   a.part_ml = reinterpret_cast<float *>(wsp + ws.cum_bytes);
   a.part_acc = reinterpret_cast<float *>(wsp + ws.cum_bytes + ws.ml_bytes);
+  a.shared_slot0 = (int64_t)ws.shared_slot0;
   a.cohort_size = cohort_size;
   a.cohort_shared_blocks = cohort_shared_blocks;
   a.dtype = dtype;

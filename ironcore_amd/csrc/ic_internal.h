@@ -61,7 +61,8 @@ struct DecodeArgs {
   int max_context_len;
   float scale;
   int min_chunk_tokens;  // smallest split-K share (multiple of block_size)
-  int32_t *cum_blocks;   // workspace: [rows + 1]
+  int32_t *cum_blocks;   // workspace: [n_seqs + 1], then [n_cohorts + 1] with cohorts
+  int64_t shared_slot0;  // first partial slot of the shared phase
   float *part_ml;        // workspace: [partial slots, 2]
   float *part_acc;       // workspace: [partial slots, hd]
   int cohort_size;       // 1 = no shared prefixes
@@ -109,39 +110,58 @@ inline int elem_size(int dtype) { return dtype == 2 ? 4 : 2; }
 // groups are cut into ceil(group / 8) sub-groups.
 inline int decode_heads_per_wave(int group) { return group <= 8 ? group : 8; }
 
-// Most (member, head) matrix columns a wave of the cohort path carries.
-constexpr int kMaxCohortColumns = 32;
+// Shared-prefix cohorts: a wave carries 16 matrix columns, i.e. the heads of
+// 16 / group members; up to 8 waves of one workgroup walk a cohort's shared
+// tiles together, each with its own members.
+constexpr int kCohortColumnsPerWave = 16;
+constexpr int kMaxCohortWaves = 8;
 
-// Work layout of one decode call: rows of tiles and matrix columns per pair.
+// Work layout of one decode call.
 struct DecodeLayout {
-  int cols;   // columns per pair (= stride of the partial arrays)
-  int nsub;   // query sub-groups per KV head
-  int rows;   // rows of the tile sequence
+  int cols;        // matrix columns per partial slot
+  int nsub;        // query sub-groups per KV head
+  int n_cohorts;   // 0 without cohorts
+  int spw;         // cohort members per wave in the shared phase
+  int unit_shift;  // log2 of the waves that share one cohort's tiles
+  bool ok;         // false: the cohort does not fit (group > 16 or too many members)
 };
 inline DecodeLayout decode_layout(int n_seqs, int hn, int gn, int cohort_size) {
   const int group = hn / gn;
   if (cohort_size <= 1) {
     const int gt = decode_heads_per_wave(group);
-    return {gt, (group + gt - 1) / gt, n_seqs};
+    return {gt, (group + gt - 1) / gt, 0, 1, 0, true};
   }
-  const int cohorts = (n_seqs + cohort_size - 1) / cohort_size;
-  return {group * cohort_size, 1, cohorts * (cohort_size + 1)};
+  if (group > kCohortColumnsPerWave) return {0, 0, 0, 0, 0, false};
+  int spw = kCohortColumnsPerWave / group;
+  if (spw > cohort_size) spw = cohort_size;
+  const int waves = (cohort_size + spw - 1) / spw;
+  int shift = 0;
+  while ((1 << shift) < waves) ++shift;
+  if ((1 << shift) > kMaxCohortWaves) return {0, 0, 0, 0, 0, false};
+  return {spw * group, 1, (n_seqs + cohort_size - 1) / cohort_size, spw, shift, true};
 }
 
 // Split-K workspace layout for the decode entry points.
 struct DecodeWorkspace {
-  size_t cum_bytes;  // int32 [rows + 1], padded to 256
-  size_t ml_bytes;   // float [slots, 2], padded to 256
-  size_t acc_bytes;  // float [slots, hd]
+  size_t cum_bytes;     // int32 [n_seqs + 1] then [n_cohorts + 1], padded to 256
+  size_t ml_bytes;      // float [slots, 2], padded to 256
+  size_t acc_bytes;     // float [slots, hd]
+  size_t shared_slot0;  // first partial slot of the shared phase
   size_t total() const { return cum_bytes + ml_bytes + acc_bytes; }
 };
 inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd, int cohort_size) {
   const DecodeLayout lay = decode_layout(n_seqs, hn, gn, cohort_size);
-  // one partial per (wave, row, pair) segment: fewer than waves + rows*pairs of them
-  const size_t slots = ((size_t)kMaxDecodeWaves + (size_t)lay.rows * gn * lay.nsub) * lay.cols;
+  const size_t pairs = (size_t)gn * lay.nsub;
+  // one partial per (wave, row, pair) segment: fewer than waves + rows*pairs of them; the shared
+  // phase has one per (unit, cohort, pair) segment and wave of the unit
+  const size_t own = (size_t)kMaxDecodeWaves + (size_t)n_seqs * pairs;
+  const size_t shared = lay.n_cohorts > 0
+                            ? (size_t)kMaxDecodeWaves + (((size_t)lay.n_cohorts * pairs) << lay.unit_shift)
+                            : 0;
+  const size_t slots = (own + shared) * lay.cols;
   auto pad = [](size_t n) { return (n + 255) & ~(size_t)255; };
-  return {pad(((size_t)lay.rows + 1) * sizeof(int32_t)), pad(slots * 2 * sizeof(float)),
-          slots * hd * sizeof(float)};
+  return {pad(((size_t)n_seqs + 1 + (size_t)lay.n_cohorts + 1) * sizeof(int32_t)),
+          pad(slots * 2 * sizeof(float)), slots * hd * sizeof(float), own};
 }
 
 // Compute units of the current device (cached per device ordinal).

@@ -79,10 +79,10 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
   const int64_t wid = (int64_t)xcd_major_workgroup() * NW + wave;
   int64_t left;  // tiles not yet consumed
   TileCursor c;
-  if (!locate_chunk<BS>(p, lane, wid, left, c)) return;
+  if (!locate_chunk<BS>(p, lane, 0, wid, left, c)) return;
   TileCursor walk = c;  // gathers tile addresses ahead of the arithmetic
   TileCursor peek = c;  // the segment after the current one (its q is prefetched)
-  next_pair<BS>(p, peek);
+  next_pair(p, GlobalRows<BS>{p, 0}, peek);
   int seg_blk0 = c.blk;
 
   uint32_t lane_off[NLD];
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
       seg_blk0 = 0;
 #pragma unroll
       for (int g = 0; g < GT; ++g) qreg[g] = qnext[g];
-      next_pair<BS>(p, peek);
+      next_pair(p, GlobalRows<BS>{p, 0}, peek);
       load_q(peek, qnext);
     }
   };
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
     // ---- window: byte offsets of the next n_win tiles, one per lane and slot ---
     const int n_win = left < kWave * SW ? (int)left : kWave * SW;
     uint32_t off_lo[SW], off_hi[SW];
-    gather_window<BS, SW, ES>(p, lane, n_win, walk, off_lo, off_hi);
+    gather_window<BS, SW, ES>(p, GlobalRows<BS>{p, 0}, lane, n_win, walk, off_lo, off_hi);
 
     auto issue = [&](int i, Vec16 *kk, Vec16 *vv) {
       const int64_t tile = window_tile_offset(off_lo, off_hi, i);
@@ -291,10 +291,11 @@ constexpr int kReduceThreads = 256;
 
 // Combine the split-K partials of one pair (a KV head's query heads of one
 // sequence).  grid = (pairs per sequence, n_seqs).  A pair's tiles in a row
-// are a contiguous run of the batch-wide sequence, so the waves that touched
+// are a contiguous run of a phase's tile sequence, so the shares that touched
 // it are first_tile / chunk .. last_tile / chunk and their partial ids follow.
-// With shared-prefix cohorts a sequence has two sources: its own row and the
-// cohort's shared row, where it owns `group` of the matrix columns.
+// With shared-prefix cohorts a sequence has two sources: its own row and its
+// cohort's row of the shared phase, where it owns `group` of the matrix
+// columns of one wave of each unit.
 // Traffic is (hd+2)*4 bytes per partial, three orders of magnitude below the
 // K/V stream; what costs time here is the chain of dependent memory round
 // trips, so the prefix sums are fetched together and every thread fetches up
@@ -309,49 +310,58 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
   const int seq = blockIdx.y;
   const int COLS = p.gt;
   const int kvh = pair_in_seq / p.nsub;
-  int row_own = seq, row_sh = -1, col0 = 0, heads, head0;
-  if (p.cohort_size == 1) {
+  const bool cohorts = p.cohort_size > 1;
+  int heads, head0, cohort = 0, col_sh = 0, wave_sh = 0;
+  if (!cohorts) {
     const int sub = pair_in_seq - kvh * p.nsub;
     head0 = kvh * p.group + sub * COLS;
     heads = (p.group - sub * COLS < COLS) ? p.group - sub * COLS : COLS;
   } else {
-    const int co = seq / p.cohort_size;
-    const int u = seq - co * p.cohort_size;
-    row_sh = co * (p.cohort_size + 1);
-    row_own = row_sh + 1 + u;
-    col0 = u * p.group;
+    cohort = seq / p.cohort_size;
+    const int u = seq - cohort * p.cohort_size;
+    wave_sh = u / p.spw;                        // the wave of a unit that carries this member
+    col_sh = (u - wave_sh * p.spw) * p.group;   // its first column there
     head0 = kvh * p.group;
     heads = p.group;
   }
-  const int cum_own = p.cum_blocks[row_own];
-  const int nb_own = p.cum_blocks[row_own + 1] - cum_own;
-  const int cum_all = p.cum_blocks[p.n_rows];
-  int cum_sh = 0, nb_sh = 0;
-  if (row_sh >= 0) {
-    cum_sh = p.cum_blocks[row_sh];
-    nb_sh = p.cum_blocks[row_sh + 1] - cum_sh;
+  const int cum_own = p.cum_blocks[seq];
+  const int nb_own = p.cum_blocks[seq + 1] - cum_own;
+  const int cum_all = p.cum_blocks[p.n_seqs];
+  int cum_sh = 0, nb_sh = 0, cum_sh_all = 0;
+  if (cohorts) {
+    cum_sh = p.cum_shared[cohort];
+    nb_sh = p.cum_shared[cohort + 1] - cum_sh;
+    cum_sh_all = p.cum_shared[p.n_cohorts];
   }
   T *orow = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)head0 * HD;
   if (nb_own + nb_sh == 0) {  // no visible token: zero rows
     for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) orow[o] = E::narrow(0.f);
     return;
   }
-  const int64_t n_tiles = (int64_t)cum_all * p.pairs_per_seq;
-  const int64_t chunk = chunk_tiles(p, n_tiles);
-  // source 0: the shared row, source 1: the sequence's own row; an empty
-  // source gets an empty wave range
-  int64_t w_lo[2], w_hi[2], slot0[2];
+  // source 0: the cohort's row of the shared phase, source 1: the sequence's
+  // own row; an empty source gets an empty share range.  A share w of a source
+  // left its partial in slot (w + slot0) * mul + add, column col0 + g.
+  int64_t w_lo[2], w_hi[2], slot0[2], mul[2], add[2];
+  int col0[2];
   {
+    const int64_t chunk = chunk_tiles(p, (int64_t)cum_sh_all * p.pairs_per_seq, phase_units(p, 1));
     const int64_t first = (int64_t)cum_sh * p.pairs_per_seq + (int64_t)pair_in_seq * nb_sh;
     w_lo[0] = first / chunk;
     w_hi[0] = nb_sh > 0 ? (first + nb_sh - 1) / chunk : w_lo[0] - 1;
-    slot0[0] = (int64_t)(row_sh < 0 ? 0 : row_sh) * p.pairs_per_seq + pair_in_seq;
+    slot0[0] = (int64_t)cohort * p.pairs_per_seq + pair_in_seq;
+    mul[0] = (int64_t)1 << p.unit_shift;
+    add[0] = p.shared_slot0 + wave_sh;
+    col0[0] = col_sh;
   }
   {
+    const int64_t chunk = chunk_tiles(p, (int64_t)cum_all * p.pairs_per_seq, phase_units(p, 0));
     const int64_t first = (int64_t)cum_own * p.pairs_per_seq + (int64_t)pair_in_seq * nb_own;
     w_lo[1] = first / chunk;
     w_hi[1] = nb_own > 0 ? (first + nb_own - 1) / chunk : w_lo[1] - 1;
-    slot0[1] = (int64_t)row_own * p.pairs_per_seq + pair_in_seq;
+    slot0[1] = (int64_t)seq * p.pairs_per_seq + pair_in_seq;
+    mul[1] = 1;
+    add[1] = 0;
+    col0[1] = 0;
   }
   // one wave covered all the sequence has for this pair and wrote the rows
   if (nb_sh == 0 && w_lo[1] == w_hi[1]) return;
@@ -368,7 +378,7 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
 #pragma unroll
         for (int u = 0; u < UB; ++u) {  // independent loads, all in flight together
           const int64_t w = wb + u <= w_hi[src] ? wb + u : w_hi[src];
-          const int64_t slot = (w + slot0[src]) * COLS + col0 + g;
+          const int64_t slot = ((w + slot0[src]) * mul[src] + add[src]) * COLS + col0[src] + g;
           ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
           av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
         }
@@ -483,14 +493,18 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.n_seqs = a.n_seqs;
   kp.hn = a.hn;
   kp.group = a.hn / a.gn;
-  if (a.cohort_size > 1 && kp.group * a.cohort_size > kMaxCohortColumns) return IC_ERR_UNSUPPORTED;
   const DecodeLayout lay = decode_layout(a.n_seqs, a.hn, a.gn, a.cohort_size);
+  if (!lay.ok) return IC_ERR_UNSUPPORTED;
   kp.nsub = lay.nsub;
   kp.gt = lay.cols;
   kp.pairs_per_seq = a.gn * lay.nsub;
-  kp.n_rows = lay.rows;
   kp.cohort_size = a.cohort_size > 1 ? a.cohort_size : 1;
   kp.cohort_shared = a.cohort_size > 1 ? a.cohort_shared_blocks : nullptr;
+  kp.n_cohorts = lay.n_cohorts;
+  kp.spw = lay.spw;
+  kp.unit_shift = lay.unit_shift;
+  kp.cum_shared = a.cum_blocks + a.n_seqs + 1;
+  kp.shared_slot0 = a.shared_slot0;
   kp.max_ctx = a.max_context_len;
   kp.n_waves = 0;
   kp.min_chunk = (a.min_chunk_tokens + 15) / 16;

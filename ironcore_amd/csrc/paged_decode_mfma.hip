@@ -1,37 +1,44 @@
 // Paged decode main kernel for 16-bit element types (bf16, fp16), on the
-// matrix cores, for any number G of query heads per KV head (1 .. 8 per wave).
+// matrix cores, for any number G of query heads per KV head (up to 16 matrix
+// columns per wave).
 //
 // Same result, same balanced split-K bookkeeping, same partial format and
 // reduce pass as paged_decode.hip.  What changes is the arithmetic of a tile:
 // with G query heads per K/V byte the vector ALU runs out of issue slots long
 // before HBM runs out of bandwidth, so both products of a 16-token tile go to
 // MFMA with the (up to 16) query heads of the pair as one matrix dimension.
-// Nothing moves between lanes and nothing goes through LDS on the per-tile
-// path:
 //
-//  * S = K . Q^T   (v_mfma_f32_16x16x32, hd/32 of them).  A = the K tile
-//    straight from the 16-byte global loads: lane l supplies row l%16 and the
-//    8 dims 32j + 8(l/16) .. +7.  B = the query rows, held in registers for
-//    the whole segment: lane l supplies head l%16 (zero beyond the pair's
-//    heads), same dims.  The result leaves lane l with the scores of head
-//    l%16 for the four S rows 4(l/16) .. +3.
-//  * S row i is token (i/4) + 4(i%4) of the tile (a lane just loads that
-//    token's K row), so lane l owns tokens kg, kg+4, kg+8, kg+12 (kg = l/16):
-//    exactly the four k-elements lane l must supply for matrix A of the next
-//    product.  exp2 and the 16-bit rounding (the reference rounds the
-//    probabilities to the element type too, attention.py:124-134) happen in
-//    place.
+//  * K and V tiles are fetched in memory order: a 16-lane group reads 256
+//    contiguous bytes of one token row.  (Fetching K straight into the matrix
+//    layout, one 16-byte piece of each of 16 rows per group, costs the L1
+//    eight times the tag look-ups and caps a cache-resident tile at 1.0 us per
+//    wave instead of 0.6.)  K then takes one hop through a wave-private LDS
+//    tile, rows padded by 16 bytes, and comes back in the matrix layout.
+//  * S = K . Q^T   (v_mfma_f32_16x16x32, hd/32 of them).  A = the K tile:
+//    lane l supplies row l%16 and the 8 dims 32j + 8(l/16) .. +7.  B = the
+//    query rows, held in registers for the whole segment: lane l supplies
+//    head l%16 (zero beyond the pair's heads), same dims.  The result leaves
+//    lane l with the scores of head l%16 for the four S rows 4(l/16) .. +3.
+//  * S row i is token (i/4) + 4(i%4) of the tile (a lane just reads that
+//    token's K row back from LDS), so lane l owns tokens kg, kg+4, kg+8, kg+12
+//    (kg = l/16): exactly the four k-elements lane l must supply for matrix A
+//    of the next product.  exp2 and the 16-bit rounding (the reference rounds
+//    the probabilities to the element type too, attention.py:124-134) happen
+//    in place.
 //  * O += P . V    (v_mfma_f32_16x16x16, one per dim owned by a lane).  B = V:
-//    lane l loads dims (l%16)*hd/16 .. of tokens kg + 4i (coalesced rows) and
-//    packs token pairs with v_perm_b32; MFMA e covers dim (l%16)*hd/16 + e.
-//    The accumulators leave lane l with heads 4kg .. 4kg+3 of those dims.
+//    lane l loads dims (l%16)*hd/16 .. of tokens kg + 4i and packs token pairs
+//    with v_perm_b32; MFMA e covers dim (l%16)*hd/16 + e.  The accumulators
+//    leave lane l with heads 4kg .. 4kg+3 of those dims.
 //  * Running maximum: a per-head reference that only moves when some score
 //    exceeds it by more than 2^5 (wave-uniform test); until then there is no
 //    cross-lane reduction and no rescale.  Row sums stay per lane and are
 //    folded once per segment.
 //
-// Per tile and wave: hd/32 + hd/16 MFMAs and about 50 vector instructions,
-// whatever G is, which leaves the kernel bound by HBM alone.
+// Per tile and wave: hd/32 + hd/16 MFMAs, about 70 vector instructions and
+// 2 * hd/32 LDS accesses, whatever G is: about 0.6 us when the tile is in the
+// cache, which leaves the kernel bound by HBM for any pool that is not.
+#include <type_traits>
+
 #include "decode_common.h"
 #include "../../include/ironcore_paged.h"
 
@@ -98,17 +105,25 @@ __device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
   return VChunk<2>{{v.x, v.y}};
 }
 
-// NCB = 16-column blocks of the query matrix a wave carries: 1 for a plain
-// pair (up to 16 heads), 2 when a shared-prefix cohort brings up to 32
-// (member, head) columns.
-template <class E, int HD, int BS, int NW, int NCB>
-// Two waves per SIMD is the design point (two 8 KiB tiles in flight each); the
-// attribute keeps the two-block variant inside 256 registers.
+// With shared-prefix cohorts the kernel runs two phases (see DecodeKP); every
+// other workgroup takes them in the opposite order, so that the LDS-fed
+// shared phase and the HBM-bound own phase overlap in time.
+// PLAN: the rows' prefix sums are laid out in LDS once per workgroup
+// (build_plan); otherwise (batches too long for LDS) every wave scans the rows.
+// COOP: a unit of the shared phase is the whole workgroup, and its waves pass
+// the shared tiles to each other through LDS: per round of NW tiles every wave
+// fetches ONE of them from memory (a full round ahead) and leaves it in its
+// slot of an LDS ring, and all waves then read each of the NW tiles back, K
+// in the matrix layout, V lane for lane.  A shared tile so crosses the memory
+// system once per workgroup instead of once per wave.
+template <class E, int HD, int BS, int NW, bool PLAN, bool COOP>
+// Two waves per SIMD is the design point (two 8 KiB tiles in flight each).
 __global__ __launch_bounds__(NW *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void paged_decode_mfma_kernel(const DecodeKP p) {
+  constexpr int NCB = 1;  // 16-column blocks of the query matrix a wave carries
   using T = typename E::type;
   constexpr int ES = 2;
-  constexpr int NK = HD / 32;  // q.k MFMAs = 16-byte K loads per lane per tile
+  constexpr int NK = HD / 32;  // q.k MFMAs = 16-byte K pieces per lane per tile
   constexpr int VE = HD / 16;  // V dims per lane = p.v MFMAs per tile
   constexpr int VW = VE / 2;   // dwords per V load
   constexpr int NT = 4;        // tokens per lane on the V side
@@ -120,10 +135,44 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
   const int n = lane & 15;   // matrix column: head (q.k) or dim group (p.v)
   const int kg = lane >> 4;  // this lane's tokens are kg, kg+4, kg+8, kg+12
 
-  const int64_t wid = (int64_t)xcd_major_workgroup() * NW + wave;
+  const int64_t wave_id = (int64_t)xcd_major_workgroup() * NW + wave;
+  const bool cohorts = p.cohort_size > 1;
+  extern __shared__ int plan_mem[];
+  PlanLds plan;
+  if constexpr (PLAN) {
+    plan = plan_carve(plan_mem, p);
+    build_plan<BS, NW * kWave>(p, plan, wave_id < NW);
+  }
+  // behind the plan: the ring of the cooperative shared phase (NW slots of one K and one V
+  // tile), then one K staging tile per wave
+  char *lds_tiles = reinterpret_cast<char *>(plan_mem + (PLAN ? ring_offset_ints(p.n_seqs, p.n_cohorts) : 0));
+  constexpr int kSlotBytes = 16 * (HD * 2 + 16) + (NT * VW / 4) * kWave * 16;  // padded K rows, then V lane by lane
+  char *xpose = lds_tiles + (COOP ? NW * kSlotBytes : 0) + wave * (16 * (HD * 2 + 16));  // this wave's K staging
+  const int n_phases = cohorts ? 2 : 1;
+  for (int phase = 0; phase < n_phases; ++phase) {
+  // 0: rows are sequences, a share per wave; 1: rows are cohorts' shared tiles, a share per unit
+  // (workgroups of one XCD go to its CUs in turn: neighbours on a CU and across CUs alternate)
+  const int order = ((blockIdx.x >> 3) ^ (blockIdx.x >> 8)) & 1;
+  const int shared = cohorts ? (phase ^ order) : 0;
+  const int64_t wid = shared ? wave_id >> p.unit_shift : wave_id;
+  const int cb_unit = shared ? (int)(wave_id & ((1 << p.unit_shift) - 1)) : 0;  // this wave's place in its unit
+  // the phase's rows
+  using Rows = typename std::conditional<PLAN, PlannedRows, GlobalRows<BS>>::type;
+  const Rows rows = [&] {
+    if constexpr (PLAN)
+      return PlannedRows{shared ? plan.cum_sh : plan.cum_own, plan.eff_sh, phase_rows(p, shared), p.cohort_size,
+                         shared};
+    else
+      return GlobalRows<BS>{p, shared};
+  }();
   int64_t left64;
   TileCursor c;
-  if (!locate_chunk<BS>(p, lane, wid, left64, c)) return;
+  bool has;
+  if constexpr (PLAN)
+    has = locate_planned(p, rows, phase_units(p, shared), lane, wid, left64, c);
+  else
+    has = locate_chunk<BS>(p, lane, shared, wid, left64, c);
+  if (!has) continue;
   // wave-uniform by construction; say so, so the bookkeeping is scalar work
   c.pair = __builtin_amdgcn_readfirstlane(c.pair);
   c.blk = __builtin_amdgcn_readfirstlane(c.blk);
@@ -135,15 +184,26 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
   // K side: S row n is token (n/4) + 4(n%4).
   const int tok_k = (n >> 2) + 4 * (n & 3);
   uint32_t k_off[NK], v_off[NT];
+  // K: piece f = 64j + lane of the tile in memory order is fetched by load j, written to LDS
+  // at kst_off[j] and read back in the matrix layout at kld_off + 64j.
+  constexpr int CPT = HD * ES / 16;     // 16-byte pieces per K row
+  constexpr int KPITCH = HD * ES + 16;  // LDS row pitch: rows 4 banks apart, reads and writes conflict-free
+  uint32_t kst_off[NK];
 #pragma unroll
-  for (int j = 0; j < NK; ++j) k_off[j] = (uint32_t)((tok_k * p.stride_token + 32 * j + 8 * kg) * ES);
+  for (int j = 0; j < NK; ++j) {
+    const int f = j * kWave + lane;
+    k_off[j] = (uint32_t)((f / CPT) * p.stride_token * ES + (f % CPT) * 16);
+    kst_off[j] = (uint32_t)((f / CPT) * KPITCH + (f % CPT) * 16);
+  }
+  const uint32_t kld_off = (uint32_t)(tok_k * KPITCH + kg * 16);
 #pragma unroll
   for (int i = 0; i < NT; ++i) v_off[i] = (uint32_t)(((kg + 4 * i) * p.stride_token + n * VE) * ES);
 
-  // Matrix column col is (member col / group, head col % group) of a cohort;
-  // a lane's columns never change, so split them once: (member << 16) | head.
+  // Shared phase: matrix column col is (member col / group of this wave's
+  // members, head col % group); a lane's columns never change, so split them
+  // once: (member << 16) | head.
   auto split = [&](int col) {
-    if (p.cohort_size == 1) return col;
+    if (!cohorts) return col;
     const int u = col / p.group;
     return (u << 16) | (col - u * p.group);
   };
@@ -157,33 +217,32 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
   // Wave-uniform facts about a segment's row and pair.
   struct Segment {
     int head0;   // first query head of the pair
-    int heads;   // query heads per member
-    int seq0;    // the row's sequence, or the cohort's first
-    int member;  // cohort rows: -1 = the shared tiles, u = member u's own tiles
+    int heads;   // query heads of the pair in this segment (own phase)
+    int seq0;    // the row's sequence; shared phase: this wave's first member
+    int seq_end; // shared phase: one past the cohort's last sequence
   };
   auto segment_of = [&](const TileCursor &tc) {
     const int kvh = tc.pair / p.nsub;
-    if (p.cohort_size == 1) {
+    if (!shared) {
       const int sub = tc.pair - kvh * p.nsub;
       const int rest = p.group - sub * COLS;
-      return Segment{kvh * p.group + sub * COLS, rest < COLS ? rest : COLS, tc.seq, -1};
+      return Segment{kvh * p.group + sub * COLS, rest < COLS ? rest : COLS, tc.seq, 0};
     }
-    const int rpc = p.cohort_size + 1;
-    const int co = tc.seq / rpc;
-    return Segment{kvh * p.group, p.group, co * p.cohort_size, tc.seq - co * rpc - 1};
+    const int first = tc.seq * p.cohort_size;
+    const int end = first + p.cohort_size < p.n_seqs ? first + p.cohort_size : p.n_seqs;
+    return Segment{kvh * p.group, p.group, first + cb_unit * p.spw, end};
   };
   Segment seg = segment_of(c);
   // Which (sequence, query head) a matrix column of the current segment is;
   // seq < 0 marks an unused column.
   auto column = [&](int col, int ug, int &seq, int &head) {
-    if (p.cohort_size == 1) {
+    if (!shared) {
       seq = col < seg.heads ? seg.seq0 : -1;
       head = seg.head0 + col;
     } else {
       const int u = ug >> 16;
       const int sq = seg.seq0 + u;
-      const bool on = u < p.cohort_size && sq < p.n_seqs && (seg.member < 0 || u == seg.member);
-      seq = on ? sq : -1;
+      seq = (u < p.spw && sq < seg.seq_end) ? sq : -1;
       head = seg.head0 + (ug & 0xffff);
     }
   };
@@ -217,9 +276,10 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
   auto finish_segment = [&]() {
     // A segment that is all a sequence has (its whole row, and no shared
     // tiles besides) writes the output rows; anything else leaves a partial.
-    const bool sole = p.cohort_size == 1 || (seg.member >= 0 && c.first == 0);
+    const bool sole = !shared && c.first == 0;
     const bool whole_pair = sole && seg_blk0 == 0 && c.blk == c.nb;
-    const int64_t partial = wid + (int64_t)c.seq * p.pairs_per_seq + c.pair;
+    int64_t partial = wid + (int64_t)c.seq * p.pairs_per_seq + c.pair;
+    if (shared) partial = p.shared_slot0 + (partial << p.unit_shift) + cb_unit;
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
       float lsum = l[cb];
@@ -267,7 +327,7 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
       for (int e = 0; e < VE; ++e) acc[cb][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
     if (left > 0) {
-      next_pair<BS>(p, c);
+      next_pair(p, rows, c);
       seg_blk0 = 0;
       seg = segment_of(c);
       fetch_q();
@@ -347,10 +407,24 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
     if (c.blk == c.nb || left == 0) finish_segment();
   };
 
+  auto k_from_lds = [&](const char *base, Vec16 *kk) {
+#pragma unroll
+    for (int j = 0; j < NK; ++j) kk[j] = *reinterpret_cast<const Vec16 *>(base + kld_off + 64 * j);
+  };
+  auto k_to_lds = [&](char *base, const Vec16 *kk) {
+#pragma unroll
+    for (int j = 0; j < NK; ++j) *reinterpret_cast<Vec16 *>(base + kst_off[j]) = kk[j];
+  };
+  auto consume_fetched = [&](Vec16 *kk, VChunk<VW> *vv) {
+    k_to_lds(xpose, kk);
+    k_from_lds(xpose, kk);
+    consume(kk, vv);
+  };
+
   while (left > 0) {
     const int n_win = left < kWave * SW ? left : kWave * SW;
     uint32_t off_lo[SW], off_hi[SW];
-    gather_window<BS, SW, ES>(p, lane, n_win, walk, off_lo, off_hi);
+    gather_window<BS, SW, ES>(p, rows, lane, n_win, walk, off_lo, off_hi);
 
     auto issue = [&](int i, Vec16 *kk, VChunk<VW> *vv) {
       const int64_t tile = window_tile_offset(off_lo, off_hi, i);
@@ -369,41 +443,122 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
     Vec16 ka[NK], kb[NK];
     VChunk<VW> va[NT], vb[NT];
     const int last = n_win - 1;
-    issue(0, ka, va);
-    for (int i = 0; i < n_win; i += 2) {
-      issue(i + 1 < last ? i + 1 : last, kb, vb);
-      consume(ka, va);
-      issue(i + 2 < last ? i + 2 : last, ka, va);
-      if (i + 1 < n_win) consume(kb, vb);
+    if (COOP && shared) {
+      // All NW waves hold the same share.  Slot w of the ring is written by wave
+      // w only, between the two barriers of a round, and read by everyone after
+      // the first: K rows as the staging tile holds them, V as lane l wrote it.
+      auto put = [&](int slot) {
+        char *base = lds_tiles + slot * kSlotBytes;
+        k_to_lds(base, ka);
+        Vec16 *dst = reinterpret_cast<Vec16 *>(base + 16 * KPITCH) + lane;
+#pragma unroll
+        for (int j = 0; j < NT * VW / 4; ++j) {
+          if constexpr (VW == 4)
+            dst[j * kWave] = Vec16{{va[j].w[0], va[j].w[1], va[j].w[2 % VW], va[j].w[3 % VW]}};
+          else
+            dst[j * kWave] = Vec16{{va[2 * j].w[0], va[2 * j].w[1], va[2 * j + 1].w[0], va[2 * j + 1].w[1]}};
+        }
+      };
+      auto get = [&](int slot) {
+        const char *base = lds_tiles + slot * kSlotBytes;
+        k_from_lds(base, kb);
+        const Vec16 *src = reinterpret_cast<const Vec16 *>(base + 16 * KPITCH) + lane;
+#pragma unroll
+        for (int j = 0; j < NT * VW / 4; ++j) {
+          const Vec16 v = src[j * kWave];
+          if constexpr (VW == 4) {
+            vb[j] = VChunk<VW>{{v.w[0], v.w[1], v.w[2 % VW], v.w[3 % VW]}};
+          } else {
+            vb[2 * j] = VChunk<VW>{{v.w[0], v.w[1]}};
+            vb[2 * j + 1] = VChunk<VW>{{v.w[2], v.w[3]}};
+          }
+        }
+      };
+      issue(wave < last ? wave : last, ka, va);
+      for (int r0 = 0; r0 < n_win; r0 += NW) {
+        put(wave);
+        __syncthreads();
+        const int mine = r0 + NW + wave;  // this wave's tile of the next round
+        issue(mine < last ? mine : last, ka, va);
+        const int here = n_win - r0 < NW ? n_win - r0 : NW;
+        for (int j = 0; j < here; ++j) {
+          get(j);
+          consume(kb, vb);
+        }
+        __syncthreads();
+      }
+    } else {
+      issue(0, ka, va);
+      for (int i = 0; i < n_win; i += 2) {
+        issue(i + 1 < last ? i + 1 : last, kb, vb);
+        consume_fetched(ka, va);
+        issue(i + 2 < last ? i + 2 : last, ka, va);
+        if (i + 1 < n_win) consume_fetched(kb, vb);
+      }
     }
   }
+  }  // phase
 }
 
-template <class E, int HD, int NCB>
-bool launch_one(DecodeKP &kp, hipStream_t stream) {
+template <class E, int HD, int NW, bool PLAN, bool COOP>
+bool launch_variant(DecodeKP &kp, size_t lds_bytes, hipStream_t stream) {
   constexpr int BS = 16;
-  constexpr int NW = kDecodeWavesPerWorkgroup;
-  static const int per_cu = [] {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, paged_decode_mfma_kernel<E, HD, BS, NW, NCB>,
-                                                     NW * kWave, 0) != hipSuccess || n < 1)
-      n = 1;
-    return n;
+  auto kernel = paged_decode_mfma_kernel<E, HD, BS, NW, PLAN, COOP>;
+  constexpr size_t kMaxLds = (PLAN ? kPlanMaxInts * sizeof(int) : 0) + tiles_lds_bytes(HD, NW, COOP);
+  static const bool ready = [&] {  // more than 64 KB of dynamic LDS has to be asked for
+    return kMaxLds <= 64 * 1024 ||
+           hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)kMaxLds) == hipSuccess;
   }();
+  if (!ready) return false;
+  // workgroups one CU holds with this much LDS (remembered for the last size asked)
+  thread_local size_t seen_bytes = ~(size_t)0;
+  thread_local int per_cu = 1;
+  if (seen_bytes != lds_bytes) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NW * kWave, lds_bytes) != hipSuccess || n < 1) n = 1;
+    per_cu = n;
+    seen_bytes = lds_bytes;
+  }
   int wgs = per_cu * device_cu_count();
   if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
   kp.n_waves = wgs * NW;
-  hipLaunchKernelGGL((paged_decode_mfma_kernel<E, HD, BS, NW, NCB>), dim3(wgs), dim3(NW * kWave), 0, stream,
-                     kp);
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(NW * kWave), lds_bytes, stream, kp);
   return true;
+}
+
+// Plain decode and cohorts one wave covers: 4-wave workgroups, no tile ring.
+// Wider cohorts: the workgroup is the unit (2, 4 or 8 waves) and shares tiles
+// through LDS.  Batches whose row bookkeeping does not fit LDS scan the rows
+// per wave and share tiles through the cache only.
+template <class E, int HD>
+bool launch_one(DecodeKP &kp, hipStream_t stream) {
+  const size_t ints = plan_ints(kp.n_seqs, kp.n_cohorts);
+  const int unit = 1 << kp.unit_shift;
+  if (ints > (size_t)kPlanMaxInts) {
+    return unit > kDecodeWavesPerWorkgroup
+               ? launch_variant<E, HD, kMaxCohortWaves, false, false>(
+                     kp, tiles_lds_bytes(HD, kMaxCohortWaves, false), stream)
+               : launch_variant<E, HD, kDecodeWavesPerWorkgroup, false, false>(
+                     kp, tiles_lds_bytes(HD, kDecodeWavesPerWorkgroup, false), stream);
+  }
+  const size_t plan_bytes = ring_offset_ints(kp.n_seqs, kp.n_cohorts) * sizeof(int);
+  switch (unit) {
+    case 1:
+      return launch_variant<E, HD, kDecodeWavesPerWorkgroup, true, false>(
+          kp, plan_bytes + tiles_lds_bytes(HD, kDecodeWavesPerWorkgroup, false), stream);
+    case 2: return launch_variant<E, HD, 2, true, true>(kp, plan_bytes + tiles_lds_bytes(HD, 2, true), stream);
+    case 4: return launch_variant<E, HD, 4, true, true>(kp, plan_bytes + tiles_lds_bytes(HD, 4, true), stream);
+    case 8: return launch_variant<E, HD, 8, true, true>(kp, plan_bytes + tiles_lds_bytes(HD, 8, true), stream);
+    default: return false;
+  }
 }
 
 template <class E>
 bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
-  const bool wide = kp.gt > 16;
   switch (hd) {
-    case 64: return wide ? launch_one<E, 64, 2>(kp, stream) : launch_one<E, 64, 1>(kp, stream);
-    case 128: return wide ? launch_one<E, 128, 2>(kp, stream) : launch_one<E, 128, 1>(kp, stream);
+    case 64: return launch_one<E, 64>(kp, stream);
+    case 128: return launch_one<E, 128>(kp, stream);
     default: return false;
   }
 }
@@ -411,7 +566,7 @@ bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
 }  // namespace
 
 bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream) {
-  if (kp.gt < 1 || kp.gt > 32) return false;
+  if (kp.gt < 1 || kp.gt > kCohortColumnsPerWave || (1 << kp.unit_shift) > kMaxCohortWaves) return false;
   switch (dtype) {
     case IC_DTYPE_BF16: return launch_hd<MfmaBf16>(kp, hd, stream);
     case IC_DTYPE_F16: return launch_hd<MfmaF16>(kp, hd, stream);

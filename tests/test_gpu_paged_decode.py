@@ -193,3 +193,20 @@ def test_decode_step_in_a_captured_graph_and_on_two_streams(gpu):
                                         wl2.max_context_len)
     torch.cuda.synchronize()
     assert torch.equal(o1, ref1) and torch.equal(o2, ref2)
+
+
+def test_decode_batch_beyond_the_lds_plan(gpu):
+    """More sequences than the row bookkeeping a workgroup keeps in LDS has room
+    for (about 12 000): the kernel variant in which every wave scans the rows
+    itself, plain and with shared-prefix cohorts."""
+    n = 13000
+    wl = workloads.make_decode_workload(n, 4, 2, 64, 1, 40, seed=21)
+    out = _run(wl, gpu)
+    _check(wl, out)
+    shared = torch.from_numpy(paged_ops.shared_prefix_blocks(wl.block_tables.numpy(), wl.context_lens.numpy(),
+                                                             wl.block_size, 16)).to(gpu)
+    d = wl.to(gpu)
+    coh = paged_ops.paged_decode(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens, d.max_context_len,
+                                 cohort_size=16, cohort_shared_blocks=shared)
+    torch.cuda.synchronize()
+    assert (coh.cpu().float() - out.float()).abs().max().item() <= 4e-3

@@ -46,8 +46,9 @@ def _check(wl, out, plain):
     assert same <= 4e-3, f"vs plain decode: max|diff| {same} ({wl.name})"
 
 
-@pytest.mark.parametrize("hn,gn,cohort", [(28, 4, 2), (28, 4, 4), (8, 8, 16), (8, 8, 32), (16, 2, 2), (16, 2, 4),
-                                         (6, 2, 5), (32, 2, 2)])
+@pytest.mark.parametrize("hn,gn,cohort", [(28, 4, 2), (28, 4, 4), (28, 4, 8), (28, 4, 16), (8, 8, 16), (8, 8, 32),
+                                         (16, 2, 2), (16, 2, 4), (16, 2, 8), (6, 2, 5), (6, 2, 3), (32, 2, 2),
+                                         (32, 2, 8), (4, 4, 100)])
 def test_grpo_groups(gpu, hn, gn, cohort):
     """Groups of samples that alias a 96-token prompt; the cohort size divides,
     equals or straddles the group size."""
@@ -121,7 +122,10 @@ def test_block_size_64(gpu):
 def test_rejects_too_many_columns_and_fp32(gpu):
     wl = workloads.make_grpo_workload(2, 8, 28, 4, 128, 32, 1, 40, seed=6)
     with pytest.raises(ValueError):
-        _run(wl, gpu, 8, shared=np.zeros(2, dtype=np.int32))  # 7 heads x 8 members > 32 columns
+        _run(wl, gpu, 17, shared=np.zeros(1, dtype=np.int32))  # 7 heads: 2 members per wave, 9 waves > 8
+    wl17 = workloads.make_grpo_workload(2, 4, 34, 2, 64, 32, 1, 40, seed=6)
+    with pytest.raises(ValueError):
+        _run(wl17, gpu, 2, shared=np.zeros(4, dtype=np.int32))  # 17 heads per KV head > 16 columns
     wl32 = workloads.make_grpo_workload(2, 4, 8, 4, 64, 32, 1, 40, dtype=torch.float32, seed=6)
     with pytest.raises(PagedLibraryError):
         _run(wl32, gpu, 2)
