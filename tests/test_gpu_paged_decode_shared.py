@@ -66,6 +66,19 @@ def test_dtypes_head_dims(gpu, dtype, hd):
     _check(wl, _run(wl, gpu, 2), plain)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("cohort", [4, 8, 16])
+def test_workgroup_wide_cohorts(gpu, dtype, hd, cohort):
+    """Cohorts that take 2, 4 and 8 waves (7 heads per KV head: two members per
+    wave): the shared tiles go through the LDS ring of a workgroup, in both
+    head dims and element types; prompts of 1 to 3 rounds of the ring and a
+    ragged last round."""
+    wl = workloads.make_grpo_workload(3, 16, 28, 4, hd, 16 * (cohort + 3), 1, 150, dtype=dtype, seed=hd + cohort)
+    plain = _run(wl, gpu, 1)
+    _check(wl, _run(wl, gpu, cohort), plain)
+
+
 def test_no_sharing_declared(gpu):
     """cohort_shared_blocks may under-state the sharing: zeros are always valid."""
     wl = workloads.make_grpo_workload(2, 4, 28, 4, 128, 64, 1, 100, seed=1)
@@ -133,10 +146,25 @@ def test_rejects_too_many_columns_and_fp32(gpu):
 
 def test_scaled_grpo_slice(gpu):
     """The GRPO benchmark shape (28 q heads, 4 kv heads, 1024-token prompt) at
-    4 prompts x 16 samples."""
+    4 prompts x 16 samples, with the cohort the benchmark uses and a narrower one."""
     wl = workloads.make_grpo_workload(4, 16, 28, 4, 128, 1024, 1, 1024, seed=0)
     plain = _run(wl, gpu, 1)
+    _check(wl, _run(wl, gpu, 16), plain)
     _check(wl, _run(wl, gpu, 4), plain)
+
+
+def test_wide_cohorts_of_unequal_prefixes_and_block_64(gpu):
+    """Members of a wide cohort alias only the blocks the helper finds equal in
+    ALL its rows: cohorts of 16 laid over groups of 4 share nothing, cohorts of
+    8 over groups of 16 share everything; 64-token pool blocks (4 tiles each)."""
+    wl = workloads.make_grpo_workload(4, 4, 28, 4, 128, 256, 1, 300, block_size=64, seed=11)
+    plain = _run(wl, gpu, 1)
+    assert _shared(wl, 16).tolist() == [0]
+    _check(wl, _run(wl, gpu, 16), plain)
+    wl = workloads.make_grpo_workload(2, 16, 28, 4, 128, 256, 1, 300, block_size=64, seed=12)
+    assert _shared(wl, 8).tolist() == [4, 4, 4, 4]
+    plain = _run(wl, gpu, 1)
+    _check(wl, _run(wl, gpu, 8), plain)
 
 
 def test_forked_samples_through_the_layer(gpu):
