@@ -42,8 +42,13 @@ rope.rope_tables / rope_rotate    pinned: float64 complex multiplication,
 gpt2.*                            pinned: cached generate == full recompute
                                   (causal-model identity); layer arithmetic vs
                                   torch.nn.functional primitives; logits and
-                                  greedy tokens vs transformers' GPT-2 on the
-                                  same random weights (tests/test_weights_hf.py).
+                                  greedy tokens vs transformers' GPT-2 and Llama
+                                  on the same random weights
+                                  (tests/test_weights_hf.py, test_weights_llama.py).
+Committed vectors                 tests/golden/*.npz (float64-loop attention
+                                  outputs; transformers' logits and greedy
+                                  continuations for seeded GPT-2 and Llama
+                                  weights), checked by tests/test_golden.py.
 _flash_attention numerics         parity unpinned (third-party flash_attn wheel,
                                   absent here; ironcore/layers/attention.py:
                                   144-206).  Not restated.
