@@ -290,7 +290,7 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
 constexpr int kReduceThreads = 256;
 
 // Combine the split-K partials of one pair (a KV head's query heads of one
-// sequence).  grid = (pairs per sequence, n_seqs).  A pair's tiles in a row
+// sequence).  grid = (pairs per sequence / pairs per workgroup, n_seqs).  A pair's tiles in a row
 // are a contiguous run of a phase's tile sequence, so the shares that touched
 // it are first_tile / chunk .. last_tile / chunk and their partial ids follow.
 // With shared-prefix cohorts a sequence has two sources: its own row and its
@@ -306,9 +306,15 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
   using T = typename E::type;
   constexpr int QPH = HD / 4;  // 4-dim groups per head row
   constexpr int UB = 4;        // partials fetched per batch
-  const int pair_in_seq = blockIdx.x;
-  const int seq = blockIdx.y;
   const int COLS = p.gt;
+  // A pair keeps COLS * QPH threads busy; a workgroup takes as many pairs of
+  // its sequence as fit (8 for MHA at hd 128), each on its own slice of threads.
+  const int width = COLS * QPH < kReduceThreads ? COLS * QPH : kReduceThreads;
+  const int per_wg = kReduceThreads / width;
+  const int tid = threadIdx.x % width;
+  const int pair_in_seq = blockIdx.x * per_wg + threadIdx.x / width;
+  const int seq = blockIdx.y;
+  if (pair_in_seq >= p.pairs_per_seq || threadIdx.x >= per_wg * width) return;
   const int kvh = pair_in_seq / p.nsub;
   const bool cohorts = p.cohort_size > 1;
   int heads, head0, cohort = 0, col_sh = 0, wave_sh = 0;
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
   }
   T *orow = reinterpret_cast<T *>(p.out) + seq * p.out_stride_seq + (int64_t)head0 * HD;
   if (nb_own + nb_sh == 0) {  // no visible token: zero rows
-    for (int o = threadIdx.x; o < heads * HD; o += kReduceThreads) orow[o] = E::narrow(0.f);
+    for (int o = tid; o < heads * HD; o += width) orow[o] = E::narrow(0.f);
     return;
   }
   // source 0: the cohort's row of the shared phase, source 1: the sequence's
@@ -365,7 +371,7 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
   }
   // one wave covered all the sequence has for this pair and wrote the rows
   if (nb_sh == 0 && w_lo[1] == w_hi[1]) return;
-  for (int o = threadIdx.x; o < heads * QPH; o += kReduceThreads) {
+  for (int o = tid; o < heads * QPH; o += width) {
     const int g = o / QPH;
     const int d = (o - g * QPH) * 4;
     float m_run = kNegInf, l_run = 0.f;
@@ -421,7 +427,9 @@ int resident_workgroups() {
 
 template <class E, int HD>
 int launch_reduce(const DecodeKP &kp, hipStream_t stream) {
-  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD>), dim3(kp.pairs_per_seq, kp.n_seqs),
+  const int width = kp.gt * (HD / 4) < kReduceThreads ? kp.gt * (HD / 4) : kReduceThreads;
+  const int per_wg = kReduceThreads / width;  // pairs per workgroup, as the kernel derives it
+  hipLaunchKernelGGL((paged_decode_reduce_kernel<E, HD>), dim3((kp.pairs_per_seq + per_wg - 1) / per_wg, kp.n_seqs),
                      dim3(kReduceThreads), 0, stream, kp);
   return hipGetLastError() == hipSuccess ? IC_OK : IC_ERR_LAUNCH;
 }
