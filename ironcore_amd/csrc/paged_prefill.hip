@@ -16,14 +16,15 @@
 //    CU, two waves per SIMD).  The wave's Q rows stay in registers as MFMA B
 //    operands.  Workgroup ids are laid out so that all tiles and heads that
 //    read the same K/V rows run on one XCD and share its L2.
-//  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Each thread
-//    fetches its 16-byte pieces through the block table TWO tiles ahead (the
-//    table entries are scalar loads issued before the step's softmax), then parks
-//    them in double-buffered LDS, row-major ([token][dim], padded pitch).
-//    Every load is unconditional (addresses are clamped into the sequence's
-//    blocks, rows past the context are zeroed when parked), so the waits on
-//    the memory counter are exact and a tile's latency hides behind two
-//    tiles of arithmetic.
+//  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Four waves stage
+//    K and four stage V, each one 16-row group of every tile: its 16-byte
+//    pieces are fetched through the block table TWO tiles ahead (one table
+//    entry per wave and tile, a scalar load issued before the step's
+//    softmax), then parked in double-buffered LDS, row-major ([token][dim],
+//    padded pitch).  Every load is unconditional (addresses are clamped into
+//    the sequence's blocks, rows past the context are zeroed when parked), so
+//    the waits on the memory counter are exact and a tile's latency hides
+//    behind two tiles of arithmetic.
 //  * Two-sided schedule: the waves of a SIMD run half a tile apart, one in
 //    its matrix step while the other is in its vector (softmax) step, with a
 //    workgroup barrier between steps; see the loop at the end of the kernel.
@@ -137,11 +138,11 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   constexpr int OB = HD / 32;          // 32-wide blocks of the output head dim
   constexpr int TB = kBN / 32;         // 32-token blocks per tile
   constexpr int CPR = HD / 8;          // 16-byte chunks per token row
-  constexpr int RPP = kPrefillThreads / CPR;         // token rows staged per pass of the workgroup
-  constexpr int NCH = kBN / RPP;                     // passes (= chunks per thread) per tile
+  constexpr int WR = kWave / CPR;      // token rows one load instruction of a wave covers
+  constexpr int NST = 16 / WR;         // loads (16-byte pieces) per lane and staged tile
   constexpr int KP = HD * 2 + 16;      // K tile pitch in bytes (bank-conflict-free b128 reads)
   constexpr int VP = HD * 2 + 64;      // V tile pitch in bytes (conflict-free transposing reads)
-  static_assert(kBN % RPP == 0 && RPP % 16 == 0, "tile staging shape");
+  static_assert(kBN == 64 && 16 % WR == 0, "tile staging shape");
 
   __shared__ __attribute__((aligned(16))) char s_k[2][kBN * KP];
   __shared__ __attribute__((aligned(16))) char s_v[2][kBN * VP];
@@ -219,65 +220,73 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int my_tiles = (my_end > 0 && q0 + wave * 32 < C) ? (my_end + kBN - 1) / kBN : 0;
 
   // ---- tile staging: global -> registers -> LDS -----------------------------------
-  // In one pass the workgroup covers RPP consecutive token rows, a wave WR of
-  // them.  Pool blocks are a power of two >= 16 rows long (or the sequence is a
-  // single block), so the rows of one wave's pass lie inside one block: table
-  // entry and base address are wave-uniform scalar work and a thread only adds
-  // a fixed offset.  Nothing here is conditional: a tile index past the sweep
-  // is clamped to the last tile, a block index past the sequence to its last
-  // block (whose 16-row groups are allocated whether filled or not), and in
-  // SINGLE mode a row past the context to the last row.
-  constexpr int WR = kWave / CPR;  // rows one wave stages per pass
-  static_assert(WR <= 16 && 16 % WR == 0, "a wave's pass must stay inside a 16-row group");
-  const int row0 = tid / CPR;
-  const int cc = tid - row0 * CPR;
-  const int row_in_wave = row0 - wave * WR;
-  const uint32_t thr_off = (uint32_t)((row_in_wave * p.stride_token + cc * 8) * 2);
+  // A wave stages one 16-row group of every tile (group wave & 3) of ONE pool:
+  // the waves of side 0 stage K, those of side 1 stage V.  Pool blocks are a
+  // power of two >= 16 rows long (or the sequence is a single block), so a
+  // group lies inside one block: one table entry and one base address per wave
+  // and tile, scalar work, and a lane only adds fixed offsets.  (A wave issues
+  // an instruction every four to five cycles whatever its kind, so the
+  // address arithmetic of the staging is paid in the same currency as the
+  // softmax beside it: with two passes over both pools per thread it cost as
+  // much as the softmax.)  Nothing here is conditional: a tile index past the
+  // sweep is clamped to the last tile, a block index past the sequence to its
+  // last block (whose 16-row groups are allocated whether filled or not), and
+  // in SINGLE mode a row past the context to the last row.
+  const int grp = wave & 3;
+  const int cc = lane % CPR;
+  const int rsub = lane / CPR;
+  const char *stage_pool = side == 0 ? p.k_pool : p.v_pool;
+  const int stage_pitch = side == 0 ? KP : VP;
+  const uint32_t thr_off = (uint32_t)((rsub * p.stride_token + cc * 8) * 2);
+  const int64_t step_off = (int64_t)WR * p.stride_token * 2;
   const int64_t head_off = (int64_t)kvh * p.stride_head;
   const int last_blk = SINGLE ? 0 : (L - 1) >> p.block_shift;
   typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
   const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
   auto clamp_tile = [&](int tile) { return tile < n_tiles ? tile : n_tiles - 1; };
-  auto lookup = [&](int tile, int32_t *ent) {
-    tile = clamp_tile(tile);
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int first = tile * kBN + i * RPP + wave * WR;  // this wave's first row of the pass
-      int blk = SINGLE ? 0 : first >> p.block_shift;
-      blk = blk < last_blk ? blk : last_blk;
-      ent[i] = table_row[blk];
-    }
+  auto lookup = [&](int tile, int32_t &ent) {
+    const int first = clamp_tile(tile) * kBN + 16 * grp;  // this wave's first row of the tile
+    int blk = SINGLE ? 0 : first >> p.block_shift;
+    blk = blk < last_blk ? blk : last_blk;
+    ent = table_row[blk];
   };
-  auto fetch_rows = [&](const char *pool, int tile, const int32_t *ent, Vec16 *st) {
-    tile = clamp_tile(tile);
+  auto fetch_rows = [&](int tile, int32_t ent, Vec16 *st) {
+    const int first = clamp_tile(tile) * kBN + 16 * grp;
+    int64_t phys = ent;
+    // A corrupt table entry must not become an out-of-pool address.
+    phys = phys < 0 ? 0 : phys;
+    phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
+    if (SINGLE) {
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int first = tile * kBN + i * RPP + wave * WR;
-      int64_t phys = ent[i];
-      // A corrupt table entry must not become an out-of-pool address.
-      phys = phys < 0 ? 0 : phys;
-      phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
-      if (SINGLE) {
-        int row = first + row_in_wave;
+      for (int i = 0; i < NST; ++i) {
+        int row = first + rsub + i * WR;
         row = row < L ? row : L - 1;
-        st[i] = load16(pool + (phys * p.stride_block + head_off + (int64_t)row * p.stride_token + cc * 8) * 2);
-      } else {
-        const int rem = first & (p.block_size - 1);
-        st[i] = load16(pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2 + thr_off);
+        st[i] = load16(stage_pool + (phys * p.stride_block + head_off + (int64_t)row * p.stride_token + cc * 8) * 2);
       }
+    } else {
+      const int rem = first & (p.block_size - 1);
+      const char *base = stage_pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2 + thr_off;
+#pragma unroll
+      for (int i = 0; i < NST; ++i) st[i] = load16(base + i * step_off);
     }
   };
-  const int park_k = row0 * KP + cc * 16;
-  const int park_v = row0 * VP + cc * 16;
-  auto park_rows = [&](char *buf, int at, int pitch, int tile, const Vec16 *st) {
+  const int park_at = (16 * grp + rsub) * stage_pitch + cc * 16;
+  auto park_rows = [&](int tile, const Vec16 *st) {
     if (tile >= n_tiles) return;
+    char *buf = (side == 0 ? s_k[tile & 1] : s_v[tile & 1]) + park_at;
+    const int row = tile * kBN + 16 * grp + rsub;
+    if (tile * kBN + 16 * grp + 16 <= L) {  // the whole group lies inside the context (wave-uniform)
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const bool live = tile * kBN + i * RPP + row0 < L;  // rows past the context are parked as zeros
-      Vec16 v;
+      for (int i = 0; i < NST; ++i) store16(buf + i * WR * stage_pitch, st[i]);
+    } else {
 #pragma unroll
-      for (int w = 0; w < 4; ++w) v.w[w] = live ? st[i].w[w] : 0u;
-      store16(buf + at + i * RPP * pitch, v);
+      for (int i = 0; i < NST; ++i) {
+        const bool live = row + i * WR < L;  // rows past the context are parked as zeros
+        Vec16 v;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v.w[w] = live ? st[i].w[w] : 0u;
+        store16(buf + i * WR * stage_pitch, v);
+      }
     }
   };
 
@@ -395,22 +404,14 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // busy at the same time.  A workgroup barrier ends each phase.
   //   side 0:  M(0) V(0) M(1) V(1) ... M(n) V(n)  -
   //   side 1:   -   M(0) V(0) M(1) ... V(n-1) M(n) V(n)
-  // LDS double buffers: K(k) and V(k-1) are read in phases 2k and 2k+1, so the
-  // pair {K(k+1), V(k)} ("pair k") is parked during those same two phases into
-  // the buffers K(k-1) and V(k-2) left; every thread parks its share at the end
-  // of its own vector step (side 1: in phase 2k, side 0: in phase 2k+1).
-  // Registers: a thread carries two pairs, pair k in set k & 1; once pair k is
-  // parked its set is refilled with pair k+2.
-  Vec16 kst[2][NCH], vst[2][NCH];
-  int32_t kent[NCH], vent[NCH];  // table entries of the pair the next refill fetches
-  auto lookup_pair = [&](int pair) {
-    lookup(pair + 1, kent);
-    lookup(pair, vent);
-  };
-  auto refill = [&](int pair, Vec16 *ks_, Vec16 *vs_) {
-    fetch_rows(p.k_pool, pair + 1, kent, ks_);
-    fetch_rows(p.v_pool, pair, vent, vs_);
-  };
+  // LDS double buffers: K(k) and V(k-1) are read in phases 2k and 2k+1, so
+  // K(k+1) and V(k) are parked during those same two phases into the buffers
+  // K(k-1) and V(k-2) left: side 1 parks V(k) at the end of its vector step of
+  // phase 2k, side 0 parks K(k+1) at the end of its vector step of phase 2k+1.
+  // Registers: a thread carries two staged tiles of its pool; once a tile is
+  // parked its set is refilled with the tile two further on.
+  Vec16 stg[2][NST];
+  int32_t ent;  // table entry of the tile the next refill fetches
   auto matrix_step = [&](int k) {
     if (k >= 1 && k <= my_tiles) weighted_values(k - 1);
     if (k < my_tiles) {
@@ -422,55 +423,66 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
         for (int i = 0; i < 16; ++i) s[tb][i] = 0.f;
     }
   };
-  auto vector_step = [&](int j, int pair, Vec16 *ks_, Vec16 *vs_) {
-    // The scalar table loads for this step's refill go first: the softmax below
-    // has no LDS or scalar-memory operation whose wait would include them.
-    lookup_pair(pair + 2);
+  // Park staged tile `tile` from `set`, refill the set with tile + 2, then the
+  // softmax of tile j.  The memory operations go first (the staged data arrived
+  // two steps ago, the table entry of the refill was looked up in the previous
+  // step) and complete behind the softmax, which has no LDS or scalar-memory
+  // operation whose wait would include them.
+  auto vector_step = [&](int j, int tile, Vec16 *set) {
+    park_rows(tile, set);
+    fetch_rows(tile + 2, ent, set);
+    lookup(tile + 3, ent);  // for the next vector step, which refills with tile + 3
     if (j >= 0 && j < my_tiles) {
       softmax(j);
     } else {
 #pragma unroll
       for (int kk = 0; kk < kBN / 16; ++kk) pb[kk] = Vec16{{0u, 0u, 0u, 0u}};
     }
-    park_rows(s_k[(pair + 1) & 1], park_k, KP, pair + 1, ks_);
-    park_rows(s_v[pair & 1], park_v, VP, pair, vs_);
-    refill(pair + 2, ks_, vs_);
   };
-  // prologue: K(0) straight into LDS, pairs 0 and 1 into the register sets
-  lookup(0, kent);
-  fetch_rows(p.k_pool, 0, kent, kst[0]);
-  park_rows(s_k[0], park_k, KP, 0, kst[0]);
-  lookup_pair(0);
-  refill(0, kst[0], vst[0]);
-  lookup_pair(1);
-  refill(1, kst[1], vst[1]);
+  // prologue: K(0) straight into LDS; side 0 then holds K(1), K(2), side 1 V(0), V(1)
+  if (side == 0) {
+    lookup(0, ent);
+    fetch_rows(0, ent, stg[0]);
+    park_rows(0, stg[0]);
+    lookup(1, ent);
+    fetch_rows(1, ent, stg[0]);
+    lookup(2, ent);
+    fetch_rows(2, ent, stg[1]);
+    lookup(3, ent);  // the first vector step parks K(1) and refills with K(3)
+  } else {
+    lookup(0, ent);
+    fetch_rows(0, ent, stg[0]);
+    lookup(1, ent);
+    fetch_rows(1, ent, stg[1]);
+    lookup(2, ent);  // the first vector step parks V(0) and refills with V(2)
+  }
   __syncthreads();
   // Both sides pass the same number of barriers.  The loops are unrolled by two
-  // so that the register set of a pair is a compile-time choice.
+  // so that the register set of a staged tile is a compile-time choice.
   const int n_steps = (n_tiles + 2) & ~1;  // steps k = 0 .. n_steps-1 cover M(0..n_tiles), rounded up to even
   if (side == 0) {
     for (int k = 0; k < n_steps; k += 2) {
       matrix_step(k);
       __syncthreads();
-      vector_step(k, k, kst[0], vst[0]);
+      vector_step(k, k + 1, stg[0]);  // parks K(k+1)
       __syncthreads();
       matrix_step(k + 1);
       __syncthreads();
-      vector_step(k + 1, k + 1, kst[1], vst[1]);
+      vector_step(k + 1, k + 2, stg[1]);
       __syncthreads();
     }
     __syncthreads();
   } else {
-    vector_step(-1, 0, kst[0], vst[0]);
+    vector_step(-1, 0, stg[0]);  // parks V(0)
     __syncthreads();
     for (int k = 0; k < n_steps; k += 2) {
       matrix_step(k);
       __syncthreads();
-      vector_step(k, k + 1, kst[1], vst[1]);
+      vector_step(k, k + 1, stg[1]);  // parks V(k+1)
       __syncthreads();
       matrix_step(k + 1);
       __syncthreads();
-      vector_step(k + 1, k + 2, kst[0], vst[0]);
+      vector_step(k + 1, k + 2, stg[0]);
       __syncthreads();
     }
   }
