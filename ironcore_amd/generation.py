@@ -30,7 +30,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from .kv_cache import PagedKVCache
-from .layers.attention import Attention
+from .layers.attention import Attention, PagedAttentionMetadata
 from .layers.module import BaseModule, get_model_dtype
 from .layers.rotary import RotaryPositionalEmbedding
 
@@ -281,12 +281,17 @@ class LanguageModel(BaseModule):
             self.embedding.word_embeddings.weight[self.vocab_size:].zero_()
 
     def forward(self, input_ids, labels=None, *, kv_cache: Optional[PagedKVCache] = None,
-                seq_ids: Optional[Sequence[int]] = None):
+                seq_ids: Optional[Sequence[int]] = None, attn_metadata=None, position_ids=None):
         if labels is not None:
             raise NotImplementedError("loss computation is a training feature")
         b, s = input_ids.shape
         dev = input_ids.device
-        if kv_cache is None:
+        if attn_metadata is not None:
+            # the caller did the cache bookkeeping itself (device-side, for a captured decode step)
+            if kv_cache is None or position_ids is None:
+                raise ValueError("attn_metadata comes with kv_cache and position_ids")
+            meta, attention_mask = attn_metadata, None
+        elif kv_cache is None:
             attention_mask = torch.tril(torch.ones(s, s, device=dev)).view(1, 1, s, s) > 0.5
             position_ids = torch.arange(s, device=dev).unsqueeze(0).expand(b, s)
             meta = None
@@ -325,17 +330,27 @@ def sample_next(logits: torch.Tensor, temperature: float = 0.0, top_k: int = 0,
 def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int, *,
              block_size: int = 16, temperature: float = 0.0, top_k: int = 0,
              eos_token_id: Optional[int] = None, generator: Optional[torch.Generator] = None,
-             kv_cache: Optional[PagedKVCache] = None, return_margins: bool = False):
+             kv_cache: Optional[PagedKVCache] = None, return_margins: bool = False,
+             use_graph: bool = False):
     """Batched generation through the block KV cache: one prefill pass over the
     prompts, then one cached decode step per new token.  Equal-length prompts
     ``[b, s]``.  Returns ``[b, s + n]`` token ids (and, on request, the per-step
     top-1/top-2 logit margins ``[b, n]``).  The next token is always chosen
-    from the last position's logits, as examples/generate_text.py:27-28 does."""
+    from the last position's logits, as examples/generate_text.py:27-28 does.
+
+    ``use_graph`` (greedy only) captures one decode step, cache bookkeeping and
+    token selection included, into a HIP graph and replays it: same tokens,
+    without the per-step launch and host work that bounds small models."""
     model.eval()
     b, s = input_ids.shape
     cfg = model.config.model
     if s + max_new_tokens > cfg.max_seq_len:
         raise ValueError("prompt + new tokens exceed the position table")
+    if use_graph:
+        if temperature != 0.0:
+            raise ValueError("use_graph selects tokens greedily (temperature 0)")
+        return _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id, kv_cache,
+                                 return_margins)
     own_cache = kv_cache is None
     if own_cache:
         per_seq = (s + max_new_tokens + block_size - 1) // block_size
@@ -365,6 +380,93 @@ def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int,
             kv_cache.free_sequence(sid)
     if return_margins:
         return tokens, torch.stack(margins, dim=1)
+    return tokens
+
+
+def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id, kv_cache, return_margins):
+    """The loop of :func:`generate` with everything a decode step needs kept on
+    the device: the sequences' blocks are reserved up front, the step derives
+    the new token's position and pool slot from the context lengths it
+    increments itself, and writes the chosen token into column ``col`` of the
+    output.  The prefill and the first decode step run eagerly (the second
+    also serves as the warm-up a capture needs); the rest are replays."""
+    b, s = input_ids.shape
+    dev = input_ids.device
+    cfg = model.config.model
+    if max_new_tokens < 1:
+        return (input_ids, input_ids.new_zeros(b, 0, dtype=torch.float32)) if return_margins else input_ids
+    own_cache = kv_cache is None
+    if own_cache:
+        per_seq = (s + max_new_tokens + block_size - 1) // block_size
+        kv_cache = PagedKVCache(cfg.num_layers, b * per_seq, block_size, cfg.num_attention_groups,
+                                cfg.d_model // cfg.num_attention_heads,
+                                next(model.parameters()).dtype, dev)
+    bs = kv_cache.block_size
+    seq_ids = [kv_cache.add_sequence() for _ in range(b)]
+    logits = model(input_ids, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
+
+    cached_at_end = s + max_new_tokens - 1                   # the last token chosen is never fed back
+    for sid in seq_ids:
+        kv_cache.reserve(sid, cached_at_end)
+    tables = kv_cache.block_table(seq_ids)
+    ctx = torch.tensor([kv_cache.length(sid) for sid in seq_ids], dtype=torch.int32, device=dev)
+    new_tokens = torch.zeros(b, max_new_tokens, dtype=torch.int64, device=dev)
+    margins = torch.zeros(b, max_new_tokens, dtype=torch.float32, device=dev) if return_margins else None
+    col = torch.zeros(1, 1, dtype=torch.int64, device=dev)
+    step_input = torch.zeros(b, 1, dtype=torch.int64, device=dev)
+    finished = torch.zeros(b, dtype=torch.bool, device=dev)
+
+    def select(logits):
+        if margins is not None:
+            top2 = torch.topk(logits.float(), 2, dim=-1)[0]
+            margins.scatter_(1, col.expand(b, 1), (top2[:, 0] - top2[:, 1]).unsqueeze(1))
+        nxt = logits.argmax(dim=-1, keepdim=True)
+        if eos_token_id is not None:
+            nxt = torch.where(finished.unsqueeze(1), torch.full_like(nxt, eos_token_id), nxt)
+            finished.logical_or_(nxt.squeeze(1) == eos_token_id)
+        new_tokens.scatter_(1, col.expand(b, 1), nxt)
+        col.add_(1)
+        step_input.copy_(nxt)
+
+    def decode_step():
+        pos = ctx.clone()                                    # the new token's position = tokens cached so far
+        ctx.add_(1)
+        block = tables.gather(1, (pos // bs).long().unsqueeze(1)).squeeze(1)
+        meta = PagedAttentionMetadata(
+            block_tables=tables, context_lens=ctx, slot_mapping=block.long() * bs + (pos % bs).long(),
+            max_context_len=cached_at_end, cu_seqlens_q=None, cohort_size=1, cohort_shared_blocks=None,
+            positions=pos)
+        step_logits = model(step_input, kv_cache=kv_cache, attn_metadata=meta,
+                            position_ids=pos.long().unsqueeze(1))[:, -1, :]
+        select(step_logits)
+
+    select(logits)
+    steps_run = 0
+    if max_new_tokens > 1:
+        decode_step()
+        steps_run = 1
+    if max_new_tokens > 2:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            decode_step()
+        for i in range(max_new_tokens - 2):
+            graph.replay()
+            steps_run += 1
+            if eos_token_id is not None and i % 8 == 7 and bool(finished.all()):
+                break
+    kv_cache.advance(seq_ids, steps_run)
+    n = steps_run + 1
+    if eos_token_id is not None:
+        # what the step-by-step loop returns: it stops right after the step at which every row has ended
+        ended = ((new_tokens[:, :n] == eos_token_id).cumsum(1) > 0).all(0)
+        if bool(ended.any()):
+            n = int(ended.int().argmax()) + 1
+    tokens = torch.cat([input_ids, new_tokens[:, :n]], dim=1)
+    if own_cache:
+        for sid in seq_ids:
+            kv_cache.free_sequence(sid)
+    if return_margins:
+        return tokens, margins[:, :n]
     return tokens
 
 

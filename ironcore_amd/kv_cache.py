@@ -152,6 +152,41 @@ class PagedKVCache:
         seq.length += 1
         return blk * bs + off
 
+    # ---- decoding without per-step host work ---------------------------------------------
+    def reserve(self, sid: int, total_length: int) -> None:
+        """Give the sequence every block it needs to grow to ``total_length``
+        tokens, and un-share the block its next token goes to, so that the
+        following appends need nothing from the host (a captured graph can
+        compute their slots on the device from :meth:`block_table`)."""
+        seq = self._seqs[sid]
+        bs = self.block_size
+        idx, off = divmod(seq.length, bs)
+        if off and self.allocator.ref_count(seq.blocks[idx]) > 1:
+            new = self.allocator.allocate()
+            old = seq.blocks[idx]
+            self.k_pools[:, new].copy_(self.k_pools[:, old])
+            self.v_pools[:, new].copy_(self.v_pools[:, old])
+            self.allocator.release(old)
+            seq.blocks[idx] = new
+        while len(seq.blocks) * bs < total_length:
+            seq.blocks.append(self.allocator.allocate())
+
+    def block_table(self, seq_ids: Sequence[int]) -> torch.Tensor:
+        """int32 ``[n, max_blocks]`` device table of all blocks the sequences
+        hold, reserved ones included (rows padded with block 0)."""
+        width = max((len(self._seqs[s].blocks) for s in seq_ids), default=1) or 1
+        table = [self._seqs[s].blocks + [0] * (width - len(self._seqs[s].blocks)) for s in seq_ids]
+        return torch.tensor(table, dtype=torch.int32, device=self.device).view(len(seq_ids), width)
+
+    def advance(self, seq_ids: Sequence[int], n_tokens: int) -> None:
+        """Record that ``n_tokens`` rows per sequence were appended into
+        reserved blocks by device-side bookkeeping."""
+        for sid in seq_ids:
+            seq = self._seqs[sid]
+            if seq.length + n_tokens > len(seq.blocks) * self.block_size:
+                raise ValueError("tokens were appended beyond the reserved blocks")
+            seq.length += n_tokens
+
     # ---- per-step metadata -----------------------------------------------------------
     def prepare(self, seq_ids: Sequence[int], new_tokens: int | Iterable[int],
                 cohort_size: int = 1) -> PagedAttentionMetadata:

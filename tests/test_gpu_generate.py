@@ -136,3 +136,59 @@ def test_multiple_choice_scoring_matches_oracle(gpu, positional):
     prompts = [i // 4 for i in range(12)]
     labels = [1 if i % 4 == 2 else 0 for i in range(12)]
     assert scoring.pick_endings(prompts, got.tolist(), labels) == scoring.pick_endings(prompts, want.tolist(), labels)
+
+
+@pytest.mark.parametrize("precision,positional,groups", [("fp32", "absolute", 4), ("fp32", "rope", 2),
+                                                         ("bf16", "absolute", 1), ("bf16", "rope", 4)])
+def test_graph_replay_generate_equals_the_step_by_step_loop(gpu, precision, positional, groups):
+    """One captured decode step (device-side cache bookkeeping, attention through
+    the C ABI, token selection) replayed for every new token: the tokens and the
+    margins of the eager loop, step for step, across block boundaries (prompt
+    of 21 with block 16, 40 new tokens); fp32 also against the CPU oracle.
+    Two generations in a row reuse nothing of the first one's graph."""
+    cfg = _small(precision, groups)
+    cfg.model.positional_embedding.type = positional
+    torch.manual_seed(0)
+    model = generation.LanguageModel(cfg, vocab_size=1000)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    model = model.to(gpu)
+    if precision == "bf16":
+        model = model.to(torch.bfloat16)
+    for seed, (b, s, n) in enumerate([(3, 21, 40), (5, 16, 3), (2, 30, 2), (1, 7, 1)]):
+        ids = torch.randint(0, 1000, (b, s), generator=torch.Generator().manual_seed(seed))
+        eager, eager_margins = generation.generate(model, ids.to(gpu), n, return_margins=True)
+        graphed, margins = generation.generate(model, ids.to(gpu), n, return_margins=True, use_graph=True)
+        torch.cuda.synchronize()
+        assert graphed.shape == (b, s + n)
+        assert torch.equal(graphed, eager), f"case {seed}"
+        assert torch.equal(margins, eager_margins), f"case {seed}"
+        if precision == "fp32" and positional == "absolute":
+            want = oracle_gpt2.generate_paged(w, _dims(cfg), ids, n)
+            assert torch.equal(graphed.cpu(), want)
+
+
+def test_graph_replay_generate_with_eos_and_a_callers_cache(gpu):
+    """End-of-sequence handling on the device (finished rows keep emitting the
+    EOS id, the result is cut where the step-by-step loop stops) and a cache the
+    caller owns: the sequences stay in it with their true lengths."""
+    from ironcore_amd.kv_cache import PagedKVCache
+    cfg = _small("fp32", 4)
+    torch.manual_seed(0)
+    model = generation.LanguageModel(cfg, vocab_size=50).to(gpu)
+    ids = torch.randint(0, 50, (4, 10), generator=torch.Generator().manual_seed(3)).to(gpu)
+    free_run = generation.generate(model, ids, 30)
+    # an id that every row emits at some step, so that the loop ends early
+    counts = torch.stack([(free_run[:, 10:] == t).any(1) for t in range(50)]).sum(1)
+    eos = int(counts.argmax())
+    eager = generation.generate(model, ids, 30, eos_token_id=eos)
+    graphed = generation.generate(model, ids, 30, eos_token_id=eos, use_graph=True)
+    torch.cuda.synchronize()
+    assert torch.equal(graphed, eager)
+    m = cfg.model
+    cache = PagedKVCache(m.num_layers, 64, 16, m.num_attention_groups, m.d_model // m.num_attention_heads,
+                         torch.float32, gpu)
+    graphed = generation.generate(model, ids, 25, kv_cache=cache, use_graph=True)
+    assert torch.equal(graphed, free_run[:, :35])
+    assert sorted(cache.length(sid) for sid in range(4)) == [34] * 4    # the last token is never fed back
+    with pytest.raises(ValueError):
+        generation.generate(model, ids, 4, temperature=0.8, use_graph=True)

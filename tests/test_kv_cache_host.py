@@ -101,3 +101,47 @@ def test_pick_endings_groups_by_prompt_and_takes_the_lowest_loss():
     labels = [0, 1, 0, 0, 0, 1]
     assert pick_endings(prompts, losses, labels) == {"metric": "accuracy", "score": 50.0}
     assert pick_endings([], [], []) == 0.0
+
+
+def test_reserve_gives_blocks_ahead_and_unshares_the_block_in_use():
+    """What a decode loop without per-step host work relies on: after
+    ``reserve`` the slots that ``prepare`` would hand out one by one can be
+    computed from ``block_table`` alone."""
+    cache = PagedKVCache(1, 16, 16, 1, 4, torch.float32, "cpu")
+    root = cache.add_sequence()
+    cache.prepare([root], 20)                               # blocks: one full, one holding 4 tokens
+    cache.k_pools[0, cache.blocks(root)[1]].fill_(7.0)
+    child = cache.fork(root)                                # full block aliased, partial one copied
+    twin = cache.add_sequence()
+    cache.prepare([twin], 16)
+    shared_partial = cache.fork(twin)                       # block-aligned: the whole block is aliased
+    for sid, total in ((child, 50), (shared_partial, 40)):
+        cache.reserve(sid, total)
+        assert len(cache.blocks(sid)) * 16 >= total
+    assert cache.blocks(child)[0] == cache.blocks(root)[0] and cache.blocks(child)[1] != cache.blocks(root)[1]
+    assert bool((cache.k_pools[0, cache.blocks(child)[1]] == 7.0).all())
+    table = cache.block_table([child, shared_partial])
+    assert table.dtype == torch.int32 and table.shape == (2, 4)
+    assert table[1].tolist() == cache.blocks(shared_partial) + [0]
+    # the slots prepare() would give for the next tokens are the table's
+    want = [int(table[0, p // 16]) * 16 + p % 16 for p in range(20, 50)]
+    got = [int(cache.prepare([child], 1).slot_mapping[0]) for _ in range(30)]
+    assert got == want
+    # and advance() is the bookkeeping of the same appends done on the device
+    cache.advance([shared_partial], 24)
+    assert cache.length(shared_partial) == 40
+    with pytest.raises(ValueError):
+        cache.advance([shared_partial], 9)                  # 49 tokens do not fit 3 blocks
+
+
+def test_reserve_copies_a_shared_block_that_is_partly_filled():
+    cache = PagedKVCache(1, 8, 16, 1, 4, torch.float32, "cpu")
+    a = cache.add_sequence()
+    cache.prepare([a], 10)
+    blk = cache.blocks(a)[0]
+    cache.allocator.share(blk)                              # someone else holds the partly filled block too
+    cache.k_pools[0, blk].fill_(3.0)
+    cache.reserve(a, 30)
+    assert cache.blocks(a)[0] != blk and cache.allocator.ref_count(blk) == 1
+    assert bool((cache.k_pools[0, cache.blocks(a)[0]] == 3.0).all())
+    assert len(cache.blocks(a)) == 2
