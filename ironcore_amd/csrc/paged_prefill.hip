@@ -166,9 +166,14 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   int seq = unit / p.gn;
   const int kvh = unit - seq * p.gn;
   const int n_seqs = p.n_units / p.gn;
+  int q_lo, L, C;
   if (n_seqs <= kWave) {
+    // (the chunk bounds travel with the context lengths, one sequence per lane: the chosen
+    // sequence's come from its lane instead of a second round trip to memory)
     const int ln = threadIdx.x & (kWave - 1);
     const int mine = ln < n_seqs ? p.context_lens[ln] : -0x7fffffff;
+    const int lo_mine = ln < n_seqs ? p.cu_seqlens_q[ln] : 0;
+    const int hi_mine = ln < n_seqs ? p.cu_seqlens_q[ln + 1] : 0;
     int rank = 0;
     for (int j = 0; j < n_seqs; ++j) {
       const int other = __builtin_amdgcn_readlane(mine, j);
@@ -177,12 +182,16 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     const uint64_t hit = __ballot(rank == seq && ln < n_seqs);
     seq = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit | (1ull << 63)));
     seq = seq < n_seqs ? seq : n_seqs - 1;
+    q_lo = __builtin_amdgcn_readlane(lo_mine, seq);
+    L = __builtin_amdgcn_readlane(mine, seq);
+    C = __builtin_amdgcn_readlane(hi_mine, seq) - q_lo;
+  } else {
+    q_lo = p.cu_seqlens_q[seq];
+    L = p.context_lens[seq];
+    C = p.cu_seqlens_q[seq + 1] - q_lo;
   }
   const int h = kvh * p.group + r / p.n_qtiles;
   const int q0 = (p.n_qtiles - 1 - r % p.n_qtiles) * kBM;
-  const int q_lo = p.cu_seqlens_q[seq];
-  int L = p.context_lens[seq];
-  int C = p.cu_seqlens_q[seq + 1] - q_lo;
   if (L < 0) L = 0;
   if (C > L) C = L;  // a chunk cannot be longer than its context
   if (q0 >= C) return;
@@ -440,21 +449,25 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     }
   };
   // prologue: K(0) straight into LDS; side 0 then holds K(1), K(2), side 1 V(0), V(1)
+  // (all table entries first, then all tiles: one round trip each, not one per tile)
   if (side == 0) {
-    lookup(0, ent);
-    fetch_rows(0, ent, stg[0]);
-    park_rows(0, stg[0]);
-    lookup(1, ent);
-    fetch_rows(1, ent, stg[0]);
-    lookup(2, ent);
-    fetch_rows(2, ent, stg[1]);
+    int32_t e0, e1, e2;
+    Vec16 first[NST];
+    lookup(0, e0);
+    lookup(1, e1);
+    lookup(2, e2);
     lookup(3, ent);  // the first vector step parks K(1) and refills with K(3)
+    fetch_rows(0, e0, first);
+    fetch_rows(1, e1, stg[0]);
+    fetch_rows(2, e2, stg[1]);
+    park_rows(0, first);
   } else {
-    lookup(0, ent);
-    fetch_rows(0, ent, stg[0]);
-    lookup(1, ent);
-    fetch_rows(1, ent, stg[1]);
+    int32_t e0, e1;
+    lookup(0, e0);
+    lookup(1, e1);
     lookup(2, ent);  // the first vector step parks V(0) and refills with V(2)
+    fetch_rows(0, e0, stg[0]);
+    fetch_rows(1, e1, stg[1]);
   }
   __syncthreads();
   // Both sides pass the same number of barriers.  The loops are unrolled by two
