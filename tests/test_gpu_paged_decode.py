@@ -210,3 +210,12 @@ def test_decode_batch_beyond_the_lds_plan(gpu):
                                  cohort_size=16, cohort_shared_blocks=shared)
     torch.cuda.synchronize()
     assert (coh.cpu().float() - out.float()).abs().max().item() <= 4e-3
+
+
+@pytest.mark.parametrize("hn,gn,dtype", [(8, 2, torch.bfloat16), (4, 4, torch.float16), (2, 1, torch.float32)])
+def test_decode_long_contexts(gpu, hn, gn, dtype):
+    """Tens of thousands of tokens per sequence: a wave's share spans many of
+    its 256-tile windows and a sequence is cut over hundreds of waves."""
+    wl = workloads.make_decode_workload(3, hn, gn, 128, 30000, 70000, dtype=dtype, seed=21)
+    _check(wl, _run(wl, gpu))
+    _check(wl, _run(wl, gpu, min_chunk_tokens=16384))     # few, long shares: many windows per share

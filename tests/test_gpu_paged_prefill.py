@@ -104,3 +104,9 @@ def test_prefill_scaled_llama7b_slice(gpu):
     """The benchmark shape at reduced batch: 32 heads, head_dim 128, prefix up to 4096, 512-token chunks."""
     wl = workloads.make_prefill_workload(2, 32, 32, 128, 0, 4096, 512, 512, seed=0)
     _check(wl, gpu)
+
+
+def test_prefill_long_prefix(gpu):
+    """A 300-token chunk behind 30 000 cached tokens (470 K/V tiles per workgroup), block size 64."""
+    wl = workloads.make_prefill_workload(2, 4, 2, 128, 30000, 30000, 300, 300, block_size=64, seed=31)
+    _check(wl, gpu)
