@@ -358,7 +358,18 @@ __device__ __forceinline__ void build_plan(const DecodeKP &p, const PlanLds &pl,
   const int tid = threadIdx.x;
   const bool cohorts = p.cohort_size > 1;
   if (cohorts) {
-    for (int c = tid; c < p.n_cohorts; c += T) pl.eff_sh[c] = cohort_shared_tiles(p, c);
+    // cohort_shared_tiles for every cohort at once: the caller's count, then the minimum over the
+    // members' whole tiles, one member per thread (all context lengths in one round trip)
+    for (int c = tid; c < p.n_cohorts; c += T) {
+      const int sh = p.cohort_shared[c] * p.tiles_per_block;
+      pl.eff_sh[c] = sh > 0 ? sh : 0;
+    }
+    __syncthreads();
+    for (int r = tid; r < p.n_seqs; r += T) {
+      int ctx = p.context_lens[r];
+      ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
+      atomicMin(&pl.eff_sh[r / p.cohort_size], ctx > 0 ? ctx / 16 : 0);
+    }
     __syncthreads();
     block_prefix_sums<T>(p.n_cohorts, [&](int c) { return pl.eff_sh[c]; }, pl.cum_sh, pl.scratch);
     block_prefix_sums<T>(p.n_seqs, [&](int r) { return seq_blocks(p, r, BS) - pl.eff_sh[r / p.cohort_size]; },
