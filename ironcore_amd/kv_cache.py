@@ -120,6 +120,8 @@ class PagedKVCache:
         (reference count up), a partly filled last block is copied so that the
         two sequences can append independently."""
         src = self._seqs[sid]
+        if src.length % self.block_size and self.allocator.num_free < 1:
+            raise OutOfBlocks("no free KV block for the copy of the partly filled block")
         child = _Sequence(length=src.length)
         full = src.length // self.block_size
         for blk in src.blocks[:full]:
@@ -134,6 +136,19 @@ class PagedKVCache:
         self._next_id += 1
         self._seqs[cid] = child
         return cid
+
+    def _blocks_needed(self, seq: _Sequence, new_tokens: int) -> int:
+        """Blocks the allocator must still give for ``new_tokens`` more tokens:
+        new ones past the blocks the sequence holds, plus the private copy of a
+        shared block that the next token would be written into."""
+        if new_tokens <= 0:
+            return 0
+        bs = self.block_size
+        need = max((seq.length + new_tokens + bs - 1) // bs - len(seq.blocks), 0)
+        idx = seq.length // bs
+        if idx < len(seq.blocks) and self.allocator.ref_count(seq.blocks[idx]) > 1:
+            need += 1
+        return need
 
     def _slot_for_append(self, seq: _Sequence) -> int:
         """Slot of the next token; allocates a block at block boundaries and
@@ -160,6 +175,9 @@ class PagedKVCache:
         compute their slots on the device from :meth:`block_table`)."""
         seq = self._seqs[sid]
         bs = self.block_size
+        need = self._blocks_needed(seq, max(total_length - seq.length, 0))
+        if need > self.allocator.num_free:
+            raise OutOfBlocks(f"{need} KV blocks needed, {self.allocator.num_free} free")
         idx, off = divmod(seq.length, bs)
         if off and self.allocator.ref_count(seq.blocks[idx]) > 1:
             new = self.allocator.allocate()
@@ -204,6 +222,13 @@ class PagedKVCache:
         if len(counts) != n:
             raise ValueError("one new-token count per sequence")
         width = max(counts) if counts else 0
+        if any(c != width for c in counts):
+            # ragged chunks: rows are padded to `width`, the kernels get true bounds
+            raise NotImplementedError("per-sequence chunk lengths must be equal within one step")
+        # all or nothing: a step that does not fit leaves every sequence as it was
+        need = sum(self._blocks_needed(self._seqs[sid], c) for sid, c in zip(seq_ids, counts))
+        if need > self.allocator.num_free:
+            raise OutOfBlocks(f"{need} KV blocks needed for this step, {self.allocator.num_free} free")
         slots, positions = [], []
         for sid, c in zip(seq_ids, counts):
             seq = self._seqs[sid]
@@ -216,9 +241,6 @@ class PagedKVCache:
         table = [self._seqs[s].blocks + [0] * (max_blocks - len(self._seqs[s].blocks)) for s in seq_ids]
         dev = self.device
         cu = None
-        if any(c != width for c in counts):
-            # ragged chunks: rows are padded to `width`, the kernels get true bounds
-            raise NotImplementedError("per-sequence chunk lengths must be equal within one step")
         shared = None
         if cohort_size > 1 and n > 0:
             from .paged_ops import shared_prefix_blocks

@@ -145,3 +145,70 @@ def test_reserve_copies_a_shared_block_that_is_partly_filled():
     assert cache.blocks(a)[0] != blk and cache.allocator.ref_count(blk) == 1
     assert bool((cache.k_pools[0, cache.blocks(a)[0]] == 3.0).all())
     assert len(cache.blocks(a)) == 2
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_cache_traffic_keeps_the_books(seed):
+    """Random appends, forks, reservations and frees: at every step a block's
+    reference count is the number of sequences that hold it, no block is both
+    free and held, a block that will be written is held by one sequence only,
+    and every sequence still reads back exactly the tokens written to it
+    (token t of sequence s is stored as the value 1000 s' + t, s' the sequence
+    that wrote it first)."""
+    import random
+    rng = random.Random(seed)
+    bs = 16
+    cache = PagedKVCache(1, 48, bs, 1, 2, torch.float32, "cpu")
+    flat = cache.k_pools[0].view(-1, 2)          # [blocks * bs, hd]: gn == 1, so slot s is row s
+    want = {}                                      # sid -> list of values, one per token
+    next_tag = [0]
+
+    def append(sid, n):
+        meta = cache.prepare([sid], n)
+        for s in meta.slot_mapping.tolist():
+            want[sid].append(float(next_tag[0]))
+            flat[s] = float(next_tag[0])
+            next_tag[0] += 1
+
+    for step in range(300):
+        live = list(want)
+        op = rng.choice(["new", "append", "append", "append", "fork", "free", "reserve"])
+        try:
+            if op == "new" or not live:
+                sid = cache.add_sequence()
+                want[sid] = []
+                append(sid, rng.randint(1, 40))
+            elif op == "append":
+                append(rng.choice(live), rng.choice([1, 1, 1, 5, 17]))
+            elif op == "fork":
+                src = rng.choice(live)
+                want[cache.fork(src)] = list(want[src])
+            elif op == "reserve":
+                sid = rng.choice(live)
+                cache.reserve(sid, cache.length(sid) + rng.randint(1, 30))
+                table = cache.block_table([sid])[0].tolist()
+                assert table[:len(cache.blocks(sid))] == cache.blocks(sid)
+                nxt = cache.length(sid)          # the block the next token goes to is this sequence's alone
+                assert cache.allocator.ref_count(cache.blocks(sid)[nxt // bs]) == 1
+            else:
+                sid = rng.choice(live)
+                cache.free_sequence(sid)
+                del want[sid]
+        except OutOfBlocks:                        # nothing may have changed; make room and go on
+            victim = rng.choice(list(want))
+            cache.free_sequence(victim)
+            del want[victim]
+        # the books
+        holders = {}
+        for sid in want:
+            assert len(cache.blocks(sid)) * bs >= cache.length(sid) == len(want[sid])
+            for blk in cache.blocks(sid):
+                holders[blk] = holders.get(blk, 0) + 1
+        for blk in range(cache.num_blocks):
+            assert cache.allocator.ref_count(blk) == holders.get(blk, 0), f"step {step} block {blk}"
+        assert cache.allocator.num_free == cache.num_blocks - len(holders)
+        # the contents
+        for sid, vals in want.items():
+            blocks = cache.blocks(sid)
+            got = [flat[blocks[t // bs] * bs + t % bs, 0].item() for t in range(len(vals))]
+            assert got == vals, f"step {step} sequence {sid}"
