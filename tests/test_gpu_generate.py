@@ -192,3 +192,69 @@ def test_graph_replay_generate_with_eos_and_a_callers_cache(gpu):
     assert sorted(cache.length(sid) for sid in range(4)) == [34] * 4    # the last token is never fed back
     with pytest.raises(ValueError):
         generation.generate(model, ids, 4, temperature=0.8, use_graph=True)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_models_teacher_forced_logits(gpu, seed):
+    """Seeded random architectures (layers, heads, KV groups, head dim, norm,
+    activation, positional scheme, bias, tied or untied output) in fp32: the
+    logits of a prefill chunk, a second chunk behind it and single cached steps
+    on the GPU against the oracle's full causal pass over the same tokens
+    (teacher forcing, so near ties in the argmax cannot hide or fake a
+    difference), and the graph-replay loop against the step-by-step loop."""
+    import random
+    from ironcore_amd.kv_cache import PagedKVCache
+    from oracle import rope as oracle_rope
+    rng = random.Random(seed)
+    hd = rng.choice([64, 128])
+    heads, groups = rng.choice([(2, 1), (2, 2), (4, 1), (4, 2), (6, 3), (8, 2)])
+    layers = rng.randint(1, 3)
+    positional = rng.choice(["absolute", "rope"])
+    ln_type = rng.choice(["layernorm", "rmsnorm"])
+    activation = rng.choice(["gelu", "relu", "swiglu", "glu"])
+    no_bias = rng.choice([False, True])
+    untie = rng.choice([False, True])
+    block = rng.choice([16, 32])
+    vocab = rng.choice([300, 1000])
+    d = heads * hd
+    cfg = ic_config.MainConfig(
+        model=ic_config.ModelConfig(d_model=d, d_ffn=2 * d, num_layers=layers, num_attention_heads=heads,
+                                    num_attention_groups=groups, head_dim=hd, max_seq_len=160,
+                                    max_position_embeddings=160, dropout_attn=0.0, dropout_embd=0.0, dropout_mlp=0.0,
+                                    precision="fp32", ln_type=ln_type, activation_type=activation, no_bias=no_bias,
+                                    untie_embed=untie,
+                                    positional_embedding=ic_config.PositionalEmbeddingConfig(type=positional)),
+        trainer=ic_config.TrainerConfig(use_flash_attn=False), init=ic_config.InitConfig(seed=seed, init_std=0.05))
+    print(f"model {seed}: {layers} layers, {heads}/{groups} heads, hd {hd}, {positional}, {ln_type}, {activation}, "
+          f"no_bias {no_bias}, untied {untie}, block {block}, vocab {vocab}", flush=True)
+    torch.manual_seed(seed)
+    model = generation.LanguageModel(cfg, vocab_size=vocab)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items() if not k.startswith("rotary_pos_emb.")}
+    m = cfg.model
+    rope = None
+    if positional == "rope":
+        rope = oracle_rope.rope_tables(hd, m.max_position_embeddings, m.positional_embedding.base)
+    dims = oracle_gpt2.Dims(layers, heads, groups, d, m.ln_eps, rope=rope, ln_type=ln_type, activation=activation)
+    b, first, second, steps = rng.randint(1, 4), rng.randint(1, 60), rng.randint(1, 40), 6
+    total = first + second + steps
+    ids = torch.randint(0, vocab, (b, total), generator=torch.Generator().manual_seed(seed))
+    want = oracle_gpt2.forward_full(w, dims, ids)
+    model = model.to(gpu).eval()
+    cache = PagedKVCache(layers, b * ((total + block - 1) // block), block, groups, hd, torch.float32, gpu)
+    sids = [cache.add_sequence() for _ in range(b)]
+    got = []
+    with torch.no_grad():
+        got.append(model(ids[:, :first].to(gpu), kv_cache=cache, seq_ids=sids))
+        got.append(model(ids[:, first:first + second].to(gpu), kv_cache=cache, seq_ids=sids))
+        for t in range(first + second, total):
+            got.append(model(ids[:, t:t + 1].to(gpu), kv_cache=cache, seq_ids=sids))
+    torch.cuda.synchronize()
+    got = torch.cat(got, dim=1).cpu()
+    scale = want.abs().max().item()
+    diff = (got - want).abs().max().item()
+    assert diff <= 2e-4 * max(scale, 1.0), f"max|logit diff| {diff} (logits up to {scale})"
+    prompt = ids[:, :first].to(gpu)
+    eager = generation.generate(model, prompt, 12, block_size=block)
+    graphed = generation.generate(model, prompt, 12, block_size=block, use_graph=True)
+    torch.cuda.synchronize()
+    assert torch.equal(eager, graphed)
