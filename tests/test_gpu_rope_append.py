@@ -161,3 +161,33 @@ def test_rotary_module_mirror(gpu):
     batch_index = torch.arange(3).repeat_interleave(5)
     want = oracle_rope.rope_rotate(x.reshape(15, 4, 64), batch_index, cos, sin).bfloat16().view(3, 5, 4, 64)
     assert _same(got, want)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_bit_exact(gpu, seed):
+    """Seeded random row counts, head layouts, element types, block sizes and
+    padding slots: the rotary append and the plain append, bit for bit."""
+    import random
+    rng = random.Random(seed)
+    dtype = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+    hn, gn = rng.choice([(1, 1), (3, 1), (8, 2), (12, 12), (28, 4), (40, 8), (5, 5)])
+    hd = rng.choice([64, 128])
+    block = rng.choice([16, 32, 64])
+    nb = rng.randint(1, 20)
+    n = rng.randint(1, nb * block)
+    print(f"append case {seed}: {n} rows, {hn}/{gn} heads, hd {hd}, {dtype}, {nb} blocks of {block}", flush=True)
+    case = list(_case(n, hn, gn, hd, dtype, seed, num_blocks=nb, block_size=block, max_pos=rng.choice([8, 300, 5000])))
+    for i in rng.sample(range(n), rng.randint(0, min(n, 5))):
+        case[5][i] = -1                                    # padding rows go nowhere
+    want_q, want_kp, want_vp = _expect(*case)
+    q, k, v, kp, vp, slots, pos, cos, sin = [t.to(gpu) for t in case]
+    plain_k, plain_v = kp.clone(), vp.clone()
+    paged_ops.rope_kv_append(q, k, v, kp, vp, slots, pos, cos, sin)
+    paged_ops.kv_append(k, v, plain_k, plain_v, slots)
+    torch.cuda.synchronize()
+    assert _same(q, want_q), "rotated query differs"
+    assert _same(kp, want_kp), "K pool differs"
+    assert _same(vp, want_vp), "V pool differs"
+    want_plain_k, want_plain_v = case[3].clone(), case[4].clone()
+    oracle_paged.kv_append(want_plain_k, want_plain_v, case[1], case[2], case[5])
+    assert _same(plain_k, want_plain_k) and _same(plain_v, want_plain_v), "plain append differs"
