@@ -209,8 +209,9 @@ class PagedKVCache:
     def prepare(self, seq_ids: Sequence[int], new_tokens: int | Iterable[int],
                 cohort_size: int = 1) -> PagedAttentionMetadata:
         """Advance each sequence by its number of new tokens (one int for all,
-        or one per sequence, padded to the longest with slot -1) and build the
-        step's metadata.  The new K/V rows must then be passed through
+        or one per sequence: the step's tensors are then ``[b, longest, ...]``
+        with the rows a sequence does not have as padding, slot -1) and build
+        the step's metadata.  The new K/V rows must then be passed through
         ``Attention.forward(..., kv_cache=cache.layer(l), attn_metadata=meta)``
         for every layer; the same metadata serves all layers.
 
@@ -222,9 +223,9 @@ class PagedKVCache:
         if len(counts) != n:
             raise ValueError("one new-token count per sequence")
         width = max(counts) if counts else 0
-        if any(c != width for c in counts):
-            # ragged chunks: rows are padded to `width`, the kernels get true bounds
-            raise NotImplementedError("per-sequence chunk lengths must be equal within one step")
+        ragged = any(c != width for c in counts)
+        if ragged and cohort_size > 1:
+            raise ValueError("cohorts are a decode feature: one new token per sequence")
         # all or nothing: a step that does not fit leaves every sequence as it was
         need = sum(self._blocks_needed(self._seqs[sid], c) for sid, c in zip(seq_ids, counts))
         if need > self.allocator.num_free:
@@ -240,7 +241,16 @@ class PagedKVCache:
         max_blocks = max((len(self._seqs[s].blocks) for s in seq_ids), default=1) or 1
         table = [self._seqs[s].blocks + [0] * (max_blocks - len(self._seqs[s].blocks)) for s in seq_ids]
         dev = self.device
-        cu = None
+        cu = chunk_rows = None
+        if ragged:
+            # rows are padded to `width` ([b, width, ...] tensors); the kernels get the true bounds
+            # and the layer packs the rows that exist
+            bounds = [0]
+            for c in counts:
+                bounds.append(bounds[-1] + c)
+            cu = torch.tensor(bounds, dtype=torch.int32, device=dev)
+            chunk_rows = torch.tensor([i * width + t for i, c in enumerate(counts) for t in range(c)],
+                                      dtype=torch.int64, device=dev)
         shared = None
         if cohort_size > 1 and n > 0:
             from .paged_ops import shared_prefix_blocks
@@ -253,4 +263,5 @@ class PagedKVCache:
             cu_seqlens_q=cu,
             cohort_size=cohort_size if shared is not None else 1,
             cohort_shared_blocks=shared,
-            positions=torch.tensor(positions, dtype=torch.int32, device=dev))
+            positions=torch.tensor(positions, dtype=torch.int32, device=dev),
+            chunk_rows=chunk_rows, max_chunk_len=width)

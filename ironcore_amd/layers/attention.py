@@ -59,6 +59,11 @@ class PagedAttentionMetadata:
     cohort_size: int = 1
     cohort_shared_blocks: Optional[torch.Tensor] = None   # int32 [ceil(b / cohort_size)]
     positions: Optional[torch.Tensor] = None   # int32 [b*sq]: index of every new token in its sequence
+    # Chunks of unequal length in one step: cu_seqlens_q holds the true bounds,
+    # chunk_rows (int64 [sum of chunk lengths]) the rows of the padded [b*sq]
+    # layout that exist, max_chunk_len the longest chunk.
+    chunk_rows: Optional[torch.Tensor] = None
+    max_chunk_len: int = 0
 
 
 class Attention(BaseModule):
@@ -144,6 +149,21 @@ class Attention(BaseModule):
                                       causal=causal, scale=1.0 / self.scale_factor)
         return out.view(b, sq, hn * hd)
 
+    def _ragged_chunks(self, query, k_pool, v_pool, meta, rows, scale):
+        """Chunks of unequal length, padded to [b, sq]: the rows that exist are
+        packed for the kernel and its output rows put back; padding rows
+        return zeros."""
+        b, sq, hn, hd = query.shape
+        packed = query.reshape(b * sq, hn, hd).index_select(0, rows)
+        if query.dtype == torch.float32:
+            got = _ragged_rows_fp32(packed, k_pool, v_pool, meta, scale)
+        else:
+            got = paged_ops.paged_prefill(packed, k_pool, v_pool, meta.block_tables, meta.context_lens,
+                                          meta.cu_seqlens_q, meta.max_chunk_len, causal=True, scale=scale)
+        out = query.new_zeros(b * sq, hn * hd)
+        out.index_copy_(0, rows, got)
+        return out.view(b, sq, hn * hd)
+
     def _dense_fp32(self, query, key, value, causal):
         """fp32 has no MFMA path: every query row runs as one decode-kernel
         sequence over the keys it may see (fp32 loads, fp32 arithmetic)."""
@@ -183,6 +203,9 @@ class Attention(BaseModule):
                                      rotary_pos_emb.cos_emb, rotary_pos_emb.sin_emb)
             query = rotated.view(b, sq, hn, hd)
         scale = 1.0 / self.scale_factor
+        rows = getattr(meta, "chunk_rows", None)
+        if rows is not None:
+            return self._ragged_chunks(query, k_pool, v_pool, meta, rows, scale)
         if sq == 1:
             cohort = meta.cohort_size if query.dtype != torch.float32 else 1
             out = paged_ops.paged_decode(query.view(b, hn, hd), k_pool, v_pool, meta.block_tables,
@@ -199,6 +222,18 @@ class Attention(BaseModule):
         out = paged_ops.paged_prefill(query.reshape(b * sq, hn, hd), k_pool, v_pool, meta.block_tables,
                                       meta.context_lens, cu, sq, causal=True, scale=scale)
         return out.view(b, sq, hn * hd)
+
+
+def _ragged_rows_fp32(query_rows, k_pool, v_pool, meta, scale):
+    """fp32 chunks of unequal length: every existing query row as one
+    decode-kernel sequence over the keys it may see."""
+    cu = meta.cu_seqlens_q.long()
+    counts = cu[1:] - cu[:-1]
+    seq_of_row = torch.repeat_interleave(torch.arange(counts.numel(), device=cu.device), counts)
+    back = (cu[1:].index_select(0, seq_of_row) - 1) - torch.arange(seq_of_row.numel(), device=cu.device)
+    ctx = (meta.context_lens.long().index_select(0, seq_of_row) - back).to(torch.int32)
+    tables = meta.block_tables.index_select(0, seq_of_row)
+    return paged_ops.paged_decode(query_rows, k_pool, v_pool, tables, ctx, meta.max_context_len, scale=scale)
 
 
 def _fp32_rows_via_decode(query, k_pool, v_pool, block_tables, context_lens, max_context_len, causal, scale):

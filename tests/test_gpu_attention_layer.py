@@ -93,3 +93,48 @@ def test_paged_prefill_then_decode_through_the_layer(gpu, dtype, precision, tol)
     bits = torch.int16 if dtype != torch.float32 else torch.int32
     assert torch.equal(cache.k_pools[0].cpu().view(bits), kp.view(bits))
     assert torch.equal(cache.v_pools[0].cpu().view(bits), vp.view(bits))
+
+
+@pytest.mark.parametrize("precision,dtype,tol", [("fp32", torch.float32, 1e-5), ("bf16", torch.bfloat16, 8e-3)])
+@pytest.mark.parametrize("rotary", [False, True])
+def test_chunks_of_unequal_length_in_one_step(gpu, precision, dtype, tol, rotary):
+    """One step that gives every sequence a chunk of its own length (0, 1, 37
+    and 90 new tokens, behind prefixes of 0 to 50) returns, row for row, what
+    each sequence gets from a step of its own in a second cache; padding rows
+    come back as zeros.  With rotary embeddings the rotation is the fused one,
+    at each token's index in its sequence."""
+    from ironcore_amd.layers.rotary import RotaryPositionalEmbedding
+    hn, gn, hd = 6, 2, 64
+    attn = Attention(_cfg(hn, gn, hd, precision)).to(gpu).eval()
+    rope = RotaryPositionalEmbedding(hd, 256).to(gpu) if rotary else None
+    caches = [PagedKVCache(1, 40, 16, gn, hd, dtype, gpu) for _ in range(2)]
+    g = torch.Generator().manual_seed(7)
+
+    def draw(*shape):
+        return torch.randn(*shape, generator=g).to(dtype).to(gpu)
+
+    prefixes, chunks = [50, 0, 17, 3], [0, 1, 37, 90]
+    sids = [[c.add_sequence() for _ in prefixes] for c in caches]
+    for i, n in enumerate(prefixes):
+        if n:
+            q, k, v = draw(1, n, hn, hd), draw(1, n, gn, hd), draw(1, n, gn, hd)
+            for c, ids in zip(caches, sids):
+                attn(q, k, v, None, kv_cache=c.layer(0), attn_metadata=c.prepare([ids[i]], n), rotary_pos_emb=rope)
+    width = max(chunks)
+    q, k, v = draw(4, width, hn, hd), draw(4, width, gn, hd), draw(4, width, gn, hd)
+    meta = caches[0].prepare(sids[0], chunks)
+    together = attn(q, k, v, None, kv_cache=caches[0].layer(0), attn_metadata=meta, rotary_pos_emb=rope)
+    torch.cuda.synchronize()
+    for i, n in enumerate(chunks):
+        assert torch.count_nonzero(together[i, n:]) == 0
+        if n == 0:
+            continue
+        alone = attn(q[i:i + 1, :n], k[i:i + 1, :n], v[i:i + 1, :n], None, kv_cache=caches[1].layer(0),
+                     attn_metadata=caches[1].prepare([sids[1][i]], n), rotary_pos_emb=rope)
+        diff = (together[i, :n].float() - alone[0].float()).abs().max().item()
+        assert diff <= tol, f"sequence {i}: max|diff| {diff}"
+    # the pools hold the same rows either way
+    for i in range(4):
+        for blk_a, blk_b in zip(caches[0].blocks(sids[0][i]), caches[1].blocks(sids[1][i])):
+            assert torch.equal(caches[0].k_pools[0, blk_a], caches[1].k_pools[0, blk_b])
+            assert torch.equal(caches[0].v_pools[0, blk_a], caches[1].v_pools[0, blk_b])

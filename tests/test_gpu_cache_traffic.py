@@ -1,7 +1,8 @@
 """Random traffic through the attention layer and the block KV cache together:
 prompts of random length prefilled in one or two chunks, batches of decode
 steps over random subsets of the live sequences (with cohorts when the batch
-is made of forks listed side by side), forks and frees in between.  The host
+is made of forks listed side by side), steps that give every sequence a chunk of
+its own length, forks and frees in between.  The host
 keeps every sequence's K/V rows; after each call the layer's output must be
 the oracle's dense attention over those rows (bars: parity_bars.py)."""
 import random
@@ -34,26 +35,32 @@ def test_random_layer_and_cache_traffic(gpu, seed, hn, gn, hd, block):
         return torch.randn(b, s, heads, hd, generator=g).bfloat16()
 
     def step(sids, s, cohort=1):
-        """s new tokens for each of sids through the layer; checks the output."""
+        """New tokens for each of sids through the layer (s: one count for all, or one per
+        sequence: rows a sequence does not have are padding); checks every output row."""
         b = len(sids)
-        q, k, v = draw(b, s, hn), draw(b, s, gn), draw(b, s, gn)
+        counts = [s] * b if isinstance(s, int) else list(s)
+        width = max(counts)
+        q, k, v = draw(b, width, hn), draw(b, width, gn), draw(b, width, gn)
         meta = cache.prepare(sids, s, cohort_size=cohort)
         out = attn(q.to(gpu), k.to(gpu), v.to(gpu), None, kv_cache=cache.layer(0), attn_metadata=meta)
         torch.cuda.synchronize()
-        for i, sid in enumerate(sids):
-            K = torch.cat([rows[sid][0], k[i]]) if sid in rows else k[i]
-            V = torch.cat([rows[sid][1], v[i]]) if sid in rows else v[i]
+        for i, (sid, c) in enumerate(zip(sids, counts)):
+            assert torch.count_nonzero(out[i, c:]) == 0, "padding rows must come back as zeros"
+            if c == 0:
+                continue
+            K = torch.cat([rows[sid][0], k[i, :c]]) if sid in rows else k[i, :c]
+            V = torch.cat([rows[sid][1], v[i, :c]]) if sid in rows else v[i, :c]
             rows[sid] = (K, V)
             t = K.shape[0]
-            causal = (torch.arange(t).unsqueeze(0) <= (t - s) + torch.arange(s).unsqueeze(1)).view(1, 1, s, t)
-            ref = dense_attention(q[i:i + 1], K.unsqueeze(0), V.unsqueeze(0), causal)
-            truth = dense_attention(q[i:i + 1].double(), K.unsqueeze(0).double(), V.unsqueeze(0).double(), causal)
-            hold(out[i:i + 1], ref, truth, torch.bfloat16, f"sequence {sid} ({t} tokens, {s} new)")
+            causal = (torch.arange(t).unsqueeze(0) <= (t - c) + torch.arange(c).unsqueeze(1)).view(1, 1, c, t)
+            ref = dense_attention(q[i:i + 1, :c], K.unsqueeze(0), V.unsqueeze(0), causal)
+            truth = dense_attention(q[i:i + 1, :c].double(), K.unsqueeze(0).double(), V.unsqueeze(0).double(), causal)
+            hold(out[i:i + 1, :c], ref, truth, torch.bfloat16, f"sequence {sid} ({t} tokens, {c} new)")
 
     calls = 0
     for it in range(60):
         live = list(rows)
-        op = rng.choice(["prompt", "decode", "decode", "decode", "group", "fork", "free"])
+        op = rng.choice(["prompt", "decode", "decode", "decode", "group", "fork", "free", "ragged"])
         try:
             if op == "prompt" or not live:
                 sid = cache.add_sequence()
@@ -62,6 +69,18 @@ def test_random_layer_and_cache_traffic(gpu, seed, hn, gn, hd, block):
                 if cut:
                     step([sid], cut)             # chunked prefill: the second chunk attends behind the first
                 step([sid], n - cut)
+                calls += 1
+            elif op == "ragged":
+                # chunks of unequal length in one step: fresh prompts beside sequences that continue
+                sids = rng.sample(live, rng.randint(0, min(len(live), 3))) + \
+                    [cache.add_sequence() for _ in range(rng.randint(1, 3))]
+                counts = [rng.choice([0, 1, 5, 40, 90]) for _ in sids]
+                if max(counts) == 0:
+                    counts[-1] = 7
+                for sid, c in zip(sids, counts):
+                    if sid not in rows and c == 0:
+                        rows[sid] = (torch.zeros(0, gn, hd).bfloat16(), torch.zeros(0, gn, hd).bfloat16())
+                step(sids, counts)
                 calls += 1
             elif op == "decode":
                 batch = rng.sample(live, rng.randint(1, min(len(live), 6)))

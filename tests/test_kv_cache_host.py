@@ -212,3 +212,23 @@ def test_random_cache_traffic_keeps_the_books(seed):
             blocks = cache.blocks(sid)
             got = [flat[blocks[t // bs] * bs + t % bs, 0].item() for t in range(len(vals))]
             assert got == vals, f"step {step} sequence {sid}"
+
+
+def test_prepare_with_chunks_of_unequal_length():
+    """One step, a chunk length per sequence: slots and positions are padded to
+    the longest chunk, the true bounds and the rows that exist come with them."""
+    cache = PagedKVCache(1, 16, 16, 1, 4, torch.float32, "cpu")
+    a, b, c = cache.add_sequence(), cache.add_sequence(), cache.add_sequence()
+    cache.prepare([a], 10)
+    meta = cache.prepare([a, b, c], [3, 0, 5])
+    assert meta.context_lens.tolist() == [13, 0, 5] and meta.max_context_len == 13
+    assert meta.cu_seqlens_q.tolist() == [0, 3, 3, 8] and meta.max_chunk_len == 5
+    assert meta.chunk_rows.tolist() == [0, 1, 2, 10, 11, 12, 13, 14]
+    slots = meta.slot_mapping.view(3, 5)
+    blk_a, blk_c = cache.blocks(a)[0], cache.blocks(c)[0]
+    assert slots[0].tolist() == [blk_a * 16 + 10, blk_a * 16 + 11, blk_a * 16 + 12, -1, -1]
+    assert slots[1].tolist() == [-1] * 5
+    assert slots[2].tolist() == [blk_c * 16 + t for t in range(5)]
+    assert meta.positions.view(3, 5)[0].tolist() == [10, 11, 12, 0, 0]
+    with pytest.raises(ValueError):
+        cache.prepare([a, b], [1, 2], cohort_size=2)
