@@ -281,7 +281,8 @@ class LanguageModel(BaseModule):
             self.embedding.word_embeddings.weight[self.vocab_size:].zero_()
 
     def forward(self, input_ids, labels=None, *, kv_cache: Optional[PagedKVCache] = None,
-                seq_ids: Optional[Sequence[int]] = None, attn_metadata=None, position_ids=None):
+                seq_ids: Optional[Sequence[int]] = None, attn_metadata=None, position_ids=None,
+                new_token_counts: Optional[Sequence[int]] = None):
         if labels is not None:
             raise NotImplementedError("loss computation is a training feature")
         b, s = input_ids.shape
@@ -299,7 +300,8 @@ class LanguageModel(BaseModule):
             if seq_ids is None or len(seq_ids) != b:
                 raise ValueError("one cache sequence id per batch row")
             past = [kv_cache.length(sid) for sid in seq_ids]
-            meta = kv_cache.prepare(seq_ids, s)
+            # new_token_counts: row i of input_ids holds that many new tokens, the rest is padding
+            meta = kv_cache.prepare(seq_ids, s if new_token_counts is None else list(new_token_counts))
             attention_mask = None
             position_ids = (torch.tensor(past, device=dev).unsqueeze(1) + torch.arange(s, device=dev).unsqueeze(0))
         x = self.embedding(input_ids, position_ids)
@@ -331,12 +333,16 @@ def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int,
              block_size: int = 16, temperature: float = 0.0, top_k: int = 0,
              eos_token_id: Optional[int] = None, generator: Optional[torch.Generator] = None,
              kv_cache: Optional[PagedKVCache] = None, return_margins: bool = False,
-             use_graph: bool = False):
+             use_graph: bool = False, prompt_lens: Optional[Sequence[int]] = None):
     """Batched generation through the block KV cache: one prefill pass over the
-    prompts, then one cached decode step per new token.  Equal-length prompts
-    ``[b, s]``.  Returns ``[b, s + n]`` token ids (and, on request, the per-step
-    top-1/top-2 logit margins ``[b, n]``).  The next token is always chosen
-    from the last position's logits, as examples/generate_text.py:27-28 does.
+    prompts, then one cached decode step per new token.  Prompts ``[b, s]``;
+    returns ``[b, s + n]`` token ids (and, on request, the per-step top-1/top-2
+    logit margins ``[b, n]``).  The next token is always chosen from the last
+    position's logits, as examples/generate_text.py:27-28 does.
+
+    ``prompt_lens``: prompts of unequal length, row i of ``input_ids`` holding
+    ``prompt_lens[i]`` tokens and then padding; they are prefilled in one step
+    and the result is a list of 1-D tensors, each prompt with its continuation.
 
     ``use_graph`` (greedy only) captures one decode step, cache bookkeeping and
     token selection included, into a HIP graph and replays it: same tokens,
@@ -346,11 +352,15 @@ def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int,
     cfg = model.config.model
     if s + max_new_tokens > cfg.max_seq_len:
         raise ValueError("prompt + new tokens exceed the position table")
+    if prompt_lens is not None:
+        prompt_lens = [int(n) for n in prompt_lens]
+        if len(prompt_lens) != b or min(prompt_lens) < 1 or max(prompt_lens) > s:
+            raise ValueError("one prompt length in [1, s] per row of input_ids")
     if use_graph:
         if temperature != 0.0:
             raise ValueError("use_graph selects tokens greedily (temperature 0)")
         return _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id, kv_cache,
-                                 return_margins)
+                                 return_margins, prompt_lens)
     own_cache = kv_cache is None
     if own_cache:
         per_seq = (s + max_new_tokens + block_size - 1) // block_size
@@ -362,8 +372,11 @@ def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int,
     margins = []
     finished = torch.zeros(b, dtype=torch.bool, device=input_ids.device)
     step_input = input_ids
-    for _ in range(max_new_tokens):
-        logits = model(step_input, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
+    for step in range(max_new_tokens):
+        if step == 0:
+            logits = _prefill_logits(model, input_ids, prompt_lens, kv_cache, seq_ids)
+        else:
+            logits = model(step_input, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
         if return_margins:
             top2 = torch.topk(logits.float(), 2, dim=-1)[0]
             margins.append(top2[:, 0] - top2[:, 1])
@@ -378,12 +391,31 @@ def generate(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int,
     if own_cache:
         for sid in seq_ids:
             kv_cache.free_sequence(sid)
+    tokens = _with_prompts(tokens, s, prompt_lens)
     if return_margins:
         return tokens, torch.stack(margins, dim=1)
     return tokens
 
 
-def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id, kv_cache, return_margins):
+def _prefill_logits(model, input_ids, prompt_lens, kv_cache, seq_ids):
+    """Logits ``[b, vocab]`` at each prompt's last token after one prefill step."""
+    if prompt_lens is None:
+        return model(input_ids, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
+    logits = model(input_ids, kv_cache=kv_cache, seq_ids=seq_ids, new_token_counts=prompt_lens)
+    last = torch.tensor(prompt_lens, device=input_ids.device) - 1
+    return logits[torch.arange(len(prompt_lens), device=input_ids.device), last]
+
+
+def _with_prompts(tokens, s, prompt_lens):
+    """``tokens`` is [b, s + n] with the new tokens behind the padded prompts:
+    with prompts of unequal length, a list of prompt + continuation per row."""
+    if prompt_lens is None:
+        return tokens
+    return [torch.cat([row[:n], row[s:]]) for row, n in zip(tokens, prompt_lens)]
+
+
+def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id, kv_cache, return_margins,
+                      prompt_lens=None):
     """The loop of :func:`generate` with everything a decode step needs kept on
     the device: the sequences' blocks are reserved up front, the step derives
     the new token's position and pool slot from the context lengths it
@@ -403,11 +435,12 @@ def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id
                                 next(model.parameters()).dtype, dev)
     bs = kv_cache.block_size
     seq_ids = [kv_cache.add_sequence() for _ in range(b)]
-    logits = model(input_ids, kv_cache=kv_cache, seq_ids=seq_ids)[:, -1, :]
+    logits = _prefill_logits(model, input_ids, prompt_lens, kv_cache, seq_ids)
 
-    cached_at_end = s + max_new_tokens - 1                   # the last token chosen is never fed back
+    # the last token chosen is never fed back
+    cached_at_end = max(kv_cache.length(sid) for sid in seq_ids) + max_new_tokens - 1
     for sid in seq_ids:
-        kv_cache.reserve(sid, cached_at_end)
+        kv_cache.reserve(sid, kv_cache.length(sid) + max_new_tokens - 1)
     tables = kv_cache.block_table(seq_ids)
     ctx = torch.tensor([kv_cache.length(sid) for sid in seq_ids], dtype=torch.int32, device=dev)
     new_tokens = torch.zeros(b, max_new_tokens, dtype=torch.int64, device=dev)
@@ -461,7 +494,7 @@ def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id
         ended = ((new_tokens[:, :n] == eos_token_id).cumsum(1) > 0).all(0)
         if bool(ended.any()):
             n = int(ended.int().argmax()) + 1
-    tokens = torch.cat([input_ids, new_tokens[:, :n]], dim=1)
+    tokens = _with_prompts(torch.cat([input_ids, new_tokens[:, :n]], dim=1), s, prompt_lens)
     if own_cache:
         for sid in seq_ids:
             kv_cache.free_sequence(sid)

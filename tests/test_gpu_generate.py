@@ -258,3 +258,37 @@ def test_random_models_teacher_forced_logits(gpu, seed):
     graphed = generation.generate(model, prompt, 12, block_size=block, use_graph=True)
     torch.cuda.synchronize()
     assert torch.equal(eager, graphed)
+
+
+@pytest.mark.parametrize("positional", ["absolute", "rope"])
+def test_generate_with_prompts_of_unequal_length(gpu, positional):
+    """Prompts of 1 to 40 tokens prefilled in one step: every row continues as
+    it does when generated alone (the oracle's loop on that prompt), step by
+    step and by graph replay."""
+    from oracle import rope as oracle_rope
+    cfg = _small("fp32", 2)
+    cfg.model.positional_embedding.type = positional
+    torch.manual_seed(0)
+    model = generation.LanguageModel(cfg, vocab_size=1000)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items() if not k.startswith("rotary_pos_emb.")}
+    m = cfg.model
+    rope = None
+    if positional == "rope":
+        rope = oracle_rope.rope_tables(m.d_model // m.num_attention_heads, m.max_position_embeddings)
+    dims = oracle_gpt2.Dims(m.num_layers, m.num_attention_heads, m.num_attention_groups, m.d_model, m.ln_eps,
+                            rope=rope)
+    lens = [1, 40, 17, 16, 33]
+    ids = torch.randint(0, 1000, (len(lens), max(lens)), generator=torch.Generator().manual_seed(4))
+    model = model.to(gpu)
+    got = generation.generate(model, ids.to(gpu), 20, prompt_lens=lens)
+    graphed, margins = generation.generate(model, ids.to(gpu), 20, prompt_lens=lens, use_graph=True,
+                                           return_margins=True)
+    torch.cuda.synchronize()
+    assert margins.shape == (len(lens), 20)
+    for i, n in enumerate(lens):
+        want, want_margins = oracle_gpt2.generate_paged(w, dims, ids[i:i + 1, :n], 20, return_margins=True)
+        assert want_margins.min().item() > 1e-4
+        assert torch.equal(got[i].cpu(), want[0]), f"prompt {i} ({n} tokens)"
+        assert torch.equal(graphed[i].cpu(), want[0]), f"prompt {i} ({n} tokens), graph replay"
+    with pytest.raises(ValueError):
+        generation.generate(model, ids.to(gpu), 4, prompt_lens=[1, 2])
