@@ -504,6 +504,53 @@ def _generate_graphed(model, input_ids, max_new_tokens, block_size, eos_token_id
 
 
 @torch.no_grad()
+def generate_samples(model: LanguageModel, prompt_ids: torch.Tensor, n_samples: int, max_new_tokens: int, *,
+                     block_size: int = 16, temperature: float = 1.0, top_k: int = 0,
+                     generator: Optional[torch.Generator] = None, kv_cache: Optional[PagedKVCache] = None):
+    """``n_samples`` continuations of every prompt (rollouts of one policy on
+    one prompt, as GRPO-style training draws them).  Each prompt ``[p, s]`` is
+    prefilled ONCE; its samples are forks of that sequence, so they alias the
+    prompt's full blocks in the pools, and every decode step runs them as
+    cohorts: the shared blocks are streamed once per cohort, not once per
+    sample.  Returns ``[p, n_samples, s + n]`` token ids.  Token selection is
+    :func:`sample_next` (examples/generate_text.py:28-37); temperature 0 gives
+    ``n_samples`` copies of the greedy continuation."""
+    model.eval()
+    p, s = prompt_ids.shape
+    cfg = model.config.model
+    if s + max_new_tokens > cfg.max_seq_len:
+        raise ValueError("prompt + new tokens exceed the position table")
+    dev = prompt_ids.device
+    own_cache = kv_cache is None
+    if own_cache:
+        shared = s // block_size
+        own = (s + max_new_tokens + block_size - 1) // block_size - shared
+        kv_cache = PagedKVCache(cfg.num_layers, p * (shared + n_samples * own), block_size,
+                                cfg.num_attention_groups, cfg.d_model // cfg.num_attention_heads,
+                                next(model.parameters()).dtype, dev)
+    roots = [kv_cache.add_sequence() for _ in range(p)]
+    logits = model(prompt_ids, kv_cache=kv_cache, seq_ids=roots)[:, -1, :]
+    seq_ids = []
+    for root in roots:                        # the samples of a prompt side by side: one cohort each
+        seq_ids += [root] + [kv_cache.fork(root) for _ in range(n_samples - 1)]
+    logits = logits.repeat_interleave(n_samples, dim=0)
+    group = cfg.num_attention_heads // cfg.num_attention_groups
+    fits = group <= 16 and n_samples <= 8 * (16 // group) and next(model.parameters()).dtype != torch.float32
+    tokens = prompt_ids.repeat_interleave(n_samples, dim=0)
+    for step in range(max_new_tokens):
+        if step:
+            meta = kv_cache.prepare(seq_ids, 1, cohort_size=n_samples if fits else 1)
+            past = torch.tensor([kv_cache.length(sid) - 1 for sid in seq_ids], device=dev).unsqueeze(1)
+            logits = model(nxt, kv_cache=kv_cache, attn_metadata=meta, position_ids=past)[:, -1, :]
+        nxt = sample_next(logits, temperature, top_k, generator)
+        tokens = torch.cat([tokens, nxt], dim=1)
+    if own_cache:
+        for sid in seq_ids:
+            kv_cache.free_sequence(sid)
+    return tokens.view(p, n_samples, s + max_new_tokens)
+
+
+@torch.no_grad()
 def generate_full_recompute(model: LanguageModel, input_ids: torch.Tensor, max_new_tokens: int):
     """The reference's loop (examples/generate_text.py:24-40) with greedy
     selection: the whole sequence goes through the model at every step."""

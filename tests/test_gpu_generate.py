@@ -292,3 +292,37 @@ def test_generate_with_prompts_of_unequal_length(gpu, positional):
         assert torch.equal(graphed[i].cpu(), want[0]), f"prompt {i} ({n} tokens), graph replay"
     with pytest.raises(ValueError):
         generation.generate(model, ids.to(gpu), 4, prompt_lens=[1, 2])
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16"])
+def test_rollout_samples_share_the_prompt(gpu, precision):
+    """n continuations per prompt from ONE prefill: forks that alias the
+    prompt's blocks, decoded in cohorts (bf16; fp32 has no cohort kernel and
+    decodes them plainly).  At temperature 0 every sample is the greedy
+    continuation of its prompt; with sampling the samples differ, stay inside
+    the vocabulary and repeat under the same generator seed."""
+    cfg = _small(precision, 2)
+    torch.manual_seed(0)
+    model = generation.LanguageModel(cfg, vocab_size=1000).to(gpu)
+    if precision == "bf16":
+        model = model.to(torch.bfloat16)
+    prompts = torch.randint(0, 1000, (3, 37), generator=torch.Generator().manual_seed(6)).to(gpu)
+    greedy = generation.generate(model, prompts, 12)
+    same = generation.generate_samples(model, prompts, 5, 12, temperature=0.0)
+    torch.cuda.synchronize()
+    assert same.shape == (3, 5, 49)
+    if precision == "fp32":
+        assert torch.equal(same, greedy.unsqueeze(1).expand(3, 5, 49))
+    else:
+        # cohorts merge partial results in another order than the plain call: a near tie may flip
+        agree = (same == greedy.unsqueeze(1)).float().mean().item()
+        assert agree > 0.9 and torch.equal(same[:, :, :38], greedy.unsqueeze(1).expand(3, 5, 49)[:, :, :38])
+    g = torch.Generator(device=gpu).manual_seed(11)
+    drawn = generation.generate_samples(model, prompts, 5, 12, temperature=1.0, top_k=50, generator=g)
+    g.manual_seed(11)
+    again = generation.generate_samples(model, prompts, 5, 12, temperature=1.0, top_k=50, generator=g)
+    torch.cuda.synchronize()
+    assert torch.equal(drawn, again)
+    assert torch.equal(drawn[:, :, :37], prompts.unsqueeze(1).expand(3, 5, 37))
+    assert int(drawn.min()) >= 0 and int(drawn.max()) < 1000
+    assert len({tuple(row.tolist()) for row in drawn[0, :, 37:]}) > 1, "samples of one prompt should differ"
