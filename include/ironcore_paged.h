@@ -59,6 +59,7 @@ extern "C" {
 #define IC_ERR_WORKSPACE     (-4)  /* workspace missing or too small             */
 #define IC_ERR_LAUNCH        (-5)  /* hipGetLastError() reported a launch failure */
 #define IC_ERR_ALIGNMENT     (-6)  /* a pointer or stride breaks the 16-byte rule */
+#define IC_ERR_STATIC_LIMIT  (-7)  /* batch too large for ic_paged_decode_static's scratch */
 
 #define IC_DTYPE_BF16 0
 #define IC_DTYPE_F16  1
@@ -205,6 +206,44 @@ int ic_paged_decode_shared(void *out, int64_t out_stride_seq,
                            int cohort_size, const int32_t *cohort_shared_blocks,
                            void *workspace, size_t workspace_bytes,
                            int dtype, void *stream);
+
+/*
+ * Paged decode that allocates nothing and takes no workspace: ic_paged_decode
+ * with the workspace (row prefix sums and split-K partials) in a static device
+ * array of IC_STATIC_SCRATCH_BYTES inside the library.  It has no counterpart
+ * in the reference; it is for callers that cannot allocate device memory and
+ * have no workspace to pass: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments, same kernels and same
+ * result as ic_paged_decode (the grid is capped at 4096 waves, which no current
+ * GPU exceeds).
+ *
+ *  - Limit: ic_paged_decode_static_scratch_bytes(n_seqs, hn, gn, hd) must not
+ *    exceed IC_STATIC_SCRATCH_BYTES, else IC_ERR_STATIC_LIMIT and nothing is
+ *    launched.  The need is 520 * (4096 + n_seqs * gn * ceil(G / 8)) * min(G, 8)
+ *    bytes at hd 128 (G = hn / gn), plus 4 * (n_seqs + 2) rounded up to 256:
+ *    21.3 MB for 128 sequences of 64 q / 8 kv heads, 22.4 MB for 512 sequences
+ *    of 28 / 4 heads, 3.2 MB for 64 sequences of 32 / 32 heads.
+ *  - Each GPU the library is used on holds the array from the first call on
+ *    that device until the process ends.  The first call on a device looks the
+ *    array's address up (hipGetSymbolAddress) and, like the first launch of any
+ *    kernel variant, must not be made under stream capture.
+ *  - Every call on a GPU uses that GPU's one array: calls that overlap in time
+ *    on one GPU (two streams, two host threads) race on the partials.  Calls
+ *    ordered on one stream are safe; nothing in the array has to be cleared
+ *    between calls (each call writes every value it later reads).
+ */
+#define IC_STATIC_SCRATCH_BYTES (32u << 20)
+size_t ic_paged_decode_static_scratch_bytes(int n_seqs, int hn, int gn, int hd);
+int ic_paged_decode_static(void *out, int64_t out_stride_seq,
+                           const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool,
+                           int64_t pool_stride_block, int64_t pool_stride_head,
+                           int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens,
+                           int n_seqs, int hn, int gn, int hd, int block_size,
+                           int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens, int dtype, void *stream);
 
 /*
  * Chunked prefill against the block KV cache: each sequence brings a chunk of

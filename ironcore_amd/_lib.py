@@ -58,6 +58,15 @@ SIGNATURES = {
         c_int, c_int, c_void_p,                 # min_chunk_tokens, cohort_size, cohort_shared_blocks
         c_void_p, c_size_t,                     # workspace, workspace_bytes
         c_int, c_void_p]),                      # dtype, stream
+    "ic_paged_decode_static_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "ic_paged_decode_static": (c_int, [
+        c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
+        c_void_p, c_void_p,                     # k_pool, v_pool
+        c_int64, c_int64, c_int64,              # pool strides
+        c_void_p, c_int64, c_void_p,            # block_tables, stride, context_lens
+        c_int, c_int, c_int, c_int, c_int,      # n_seqs, hn, gn, hd, block_size
+        c_int64, c_int, c_float,                # num_blocks, max_context_len, scale
+        c_int, c_int, c_void_p]),               # min_chunk_tokens, dtype, stream
     "ic_paged_prefill": (c_int, [
         c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
         c_void_p, c_void_p,                     # k_pool, v_pool

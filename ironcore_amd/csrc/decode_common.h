@@ -35,6 +35,7 @@ struct DecodeKP {
   int pairs_per_seq;  // gn * nsub
   int max_ctx;
   int n_waves;      // waves in the main kernel's grid
+  int max_waves;    // most waves the partial arrays have slots for (host side: caps the grid)
   int min_chunk;    // smallest chunk, in tiles
   int tiles_per_block;  // 16-token tiles in one pool block (1 for block_size 16)
   float scale_log2e;

@@ -5,7 +5,35 @@
 #include "ic_internal.h"
 #include "../../include/ironcore_paged.h"
 
+// Device memory of the entry point that may not allocate (ic_paged_decode_static): the decode
+// workspace (row prefix sums and split-K partials) lives in this array instead of a buffer the
+// caller brings.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends; host code reaches it only through the address hipGetSymbolAddress returns for the
+// current device (static_scratch below), never through the array's name.
+static __device__ __align__(256) unsigned char scratch[IC_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+// Grid cap of the static entry point: 8 waves on each of up to 512 CUs (an MI355X launch uses
+// 2048).  It bounds the partial slots, so that the BASELINE decode shapes fit the scratch array.
+constexpr int kStaticMaxWaves = 4096;
+constexpr int kMaxDevices = 64;
+
+// Address of `scratch` on the current device, looked up once per device; nullptr on failure.
+void *static_scratch() {
+  static std::atomic<void *> addr[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void *p = addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    addr[dev].store(p, std::memory_order_release);
+  }
+  return p;
+}
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 bool dtype_ok(int dtype) { return dtype == IC_DTYPE_BF16 || dtype == IC_DTYPE_F16 || dtype == IC_DTYPE_F32; }
@@ -26,6 +54,72 @@ int resolve_min_chunk(int min_chunk_tokens) {
   if (min_chunk_tokens == 0) min_chunk_tokens = ic::kDefaultMinChunkTokens;
   if (min_chunk_tokens < 16 || min_chunk_tokens % 16 != 0) return -1;
   return min_chunk_tokens;
+}
+
+// Both decode entry points and the variant on the library's own scratch: checks, then the launch.
+// The workspace has partial slots for a grid of at most `max_waves` waves.
+int decode_checked(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
+                   const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                   int64_t pool_stride_head, int64_t pool_stride_token, const int32_t *block_tables,
+                   int64_t block_table_stride, const int32_t *context_lens, int n_seqs, int hn, int gn,
+                   int hd, int block_size, int64_t num_blocks, int max_context_len, float scale,
+                   int min_chunk_tokens, int cohort_size, const int32_t *cohort_shared_blocks,
+                   void *workspace, size_t workspace_bytes, int max_waves, int dtype, void *stream) {
+  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0 || cohort_size < 1)
+    return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                          num_blocks, es))
+    return rc;
+  if (n_seqs == 0) return IC_OK;
+  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
+  if (cohort_size > 1) {
+    if (!cohort_shared_blocks) return IC_ERR_NULL_POINTER;
+    if (dtype == IC_DTYPE_F32 || !ic::decode_layout(n_seqs, hn, gn, cohort_size).ok) return IC_ERR_UNSUPPORTED;
+  }
+  if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
+  if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
+  const int mc = resolve_min_chunk(min_chunk_tokens);
+  if (mc < 0) return IC_ERR_BAD_SHAPE;
+  const int64_t need_blocks = ((int64_t)max_context_len + block_size - 1) / block_size;
+  if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !stride16(q_stride_seq, es))
+    return IC_ERR_ALIGNMENT;
+  // the matrix-core kernel stores 8- or 16-byte pieces of output rows
+  if (es == 2 && (!aligned16(out) || !stride16(out_stride_seq, es))) return IC_ERR_ALIGNMENT;
+  const ic::DecodeWorkspace ws = ic::decode_workspace(n_seqs, hn, gn, hd, cohort_size, max_waves);
+  if (!workspace || workspace_bytes < ws.total() || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return IC_ERR_WORKSPACE;
+
+  ic::DecodeArgs a;
+  a.out = out;
+  a.out_stride_seq = out_stride_seq;
+  a.q = q;
+  a.q_stride_seq = q_stride_seq;
+  a.k_pool = k_pool;
+  a.v_pool = v_pool;
+  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
+  a.block_tables = block_tables;
+  a.block_table_stride = block_table_stride;
+  a.context_lens = context_lens;
+  a.n_seqs = n_seqs;
+  a.hn = hn;
+  a.gn = gn;
+  a.hd = hd;
+  a.max_context_len = max_context_len;
+  a.scale = scale;
+  a.min_chunk_tokens = mc;
+  char *wsp = static_cast<char *>(workspace);
+  a.cum_blocks = reinterpret_cast<int32_t *>(wsp);
+  a.part_ml = reinterpret_cast<float *>(wsp + ws.cum_bytes);
+  a.part_acc = reinterpret_cast<float *>(wsp + ws.cum_bytes + ws.ml_bytes);
+  a.shared_slot0 = (int64_t)ws.shared_slot0;
+  a.cohort_size = cohort_size;
+  a.cohort_shared_blocks = cohort_shared_blocks;
+  a.max_waves = max_waves;
+  a.dtype = dtype;
+  return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
 }
 
 }  // namespace
@@ -60,6 +154,9 @@ const char *ic_error_string(int code) {
     case IC_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case IC_ERR_LAUNCH: return "kernel launch failed";
     case IC_ERR_ALIGNMENT: return "pointer or stride is not 16-byte aligned";
+    case IC_ERR_STATIC_LIMIT:
+      return "the batch needs more scratch than the library's static buffer holds (IC_STATIC_SCRATCH_BYTES); "
+             "use ic_paged_decode with a caller-provided workspace";
     default: return "unknown error code";
   }
 }
@@ -182,60 +279,40 @@ int ic_paged_decode_shared(void *out, int64_t out_stride_seq, const void *q, int
                            int block_size, int64_t num_blocks, int max_context_len, float scale,
                            int min_chunk_tokens, int cohort_size, const int32_t *cohort_shared_blocks,
                            void *workspace, size_t workspace_bytes, int dtype, void *stream) {
-  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0 || cohort_size < 1)
-    return IC_ERR_BAD_SHAPE;
-  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
-  const int es = ic::elem_size(dtype);
-  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
-                          num_blocks, es))
-    return rc;
-  if (n_seqs == 0) return IC_OK;
-  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens) return IC_ERR_NULL_POINTER;
-  if (cohort_size > 1) {
-    if (!cohort_shared_blocks) return IC_ERR_NULL_POINTER;
-    if (dtype == IC_DTYPE_F32 || !ic::decode_layout(n_seqs, hn, gn, cohort_size).ok) return IC_ERR_UNSUPPORTED;
-  }
-  if (out_stride_seq < (int64_t)hn * hd || q_stride_seq < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
-  if (max_context_len == 0) max_context_len = 1;  // all-empty batch: the reduce pass writes zeros
-  const int mc = resolve_min_chunk(min_chunk_tokens);
-  if (mc < 0) return IC_ERR_BAD_SHAPE;
-  const int64_t need_blocks = ((int64_t)max_context_len + block_size - 1) / block_size;
-  if (block_table_stride < need_blocks) return IC_ERR_BAD_SHAPE;
-  if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !stride16(q_stride_seq, es))
-    return IC_ERR_ALIGNMENT;
-  // the matrix-core kernel stores 8- or 16-byte pieces of output rows
-  if (es == 2 && (!aligned16(out) || !stride16(out_stride_seq, es))) return IC_ERR_ALIGNMENT;
-  const ic::DecodeWorkspace ws = ic::decode_workspace(n_seqs, hn, gn, hd, cohort_size);
-  if (!workspace || workspace_bytes < ws.total() || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-    return IC_ERR_WORKSPACE;
+  return decode_checked(out, out_stride_seq, q, q_stride_seq, k_pool, v_pool, pool_stride_block,
+                        pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                        context_lens, n_seqs, hn, gn, hd, block_size, num_blocks, max_context_len,
+                        scale, min_chunk_tokens, cohort_size, cohort_shared_blocks, workspace,
+                        workspace_bytes, ic::kMaxDecodeWaves, dtype, stream);
+}
 
-  ic::DecodeArgs a;
-  a.out = out;
-  a.out_stride_seq = out_stride_seq;
-  a.q = q;
-  a.q_stride_seq = q_stride_seq;
-  a.k_pool = k_pool;
-  a.v_pool = v_pool;
-  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
-  a.block_tables = block_tables;
-  a.block_table_stride = block_table_stride;
-  a.context_lens = context_lens;
-  a.n_seqs = n_seqs;
-  a.hn = hn;
-  a.gn = gn;
-  a.hd = hd;
-  a.max_context_len = max_context_len;
-  a.scale = scale;
-  a.min_chunk_tokens = mc;
-  char *wsp = static_cast<char *>(workspace);
-  a.cum_blocks = reinterpret_cast<int32_t *>(wsp);
-  a.part_ml = reinterpret_cast<float *>(wsp + ws.cum_bytes);
-  a.part_acc = reinterpret_cast<float *>(wsp + ws.cum_bytes + ws.ml_bytes);
-  a.shared_slot0 = (int64_t)ws.shared_slot0;
-  a.cohort_size = cohort_size;
-  a.cohort_shared_blocks = cohort_shared_blocks;
-  a.dtype = dtype;
-  return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
+size_t ic_paged_decode_static_scratch_bytes(int n_seqs, int hn, int gn, int hd) {
+  if (n_seqs <= 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0) return 0;
+  return ic::decode_workspace(n_seqs, hn, gn, hd, 1, kStaticMaxWaves).total();
+}
+
+int ic_paged_decode_static(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                           int64_t pool_stride_head, int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens, int n_seqs, int hn, int gn, int hd,
+                           int block_size, int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens, int dtype, void *stream) {
+  if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || hd <= 0) return IC_ERR_BAD_SHAPE;
+  size_t need = 0;
+  if (n_seqs > 0) {
+    need = ic_paged_decode_static_scratch_bytes(n_seqs, hn, gn, hd);
+    if (need == 0 || need > (size_t)IC_STATIC_SCRATCH_BYTES) return IC_ERR_STATIC_LIMIT;
+  }
+  void *ws = n_seqs > 0 ? static_scratch() : nullptr;  // an empty batch launches nothing
+  if (n_seqs > 0 && ws == nullptr) return IC_ERR_LAUNCH;
+  // Nothing in the workspace has to start at zero: the main kernel writes the prefix sums and
+  // every partial the reduce pass reads, so a previous call's leftovers are never looked at.
+  return decode_checked(out, out_stride_seq, q, q_stride_seq, k_pool, v_pool, pool_stride_block,
+                        pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                        context_lens, n_seqs, hn, gn, hd, block_size, num_blocks, max_context_len,
+                        scale, min_chunk_tokens, 1, nullptr, ws, (size_t)IC_STATIC_SCRATCH_BYTES,
+                        kStaticMaxWaves, dtype, stream);
 }
 
 int ic_paged_prefill(void *out, int64_t out_stride_token, const void *q, int64_t q_stride_token,

@@ -67,6 +67,7 @@ struct DecodeArgs {
   float *part_acc;       // workspace: [partial slots, hd]
   int cohort_size;       // 1 = no shared prefixes
   const int32_t *cohort_shared_blocks;  // [ceil(n_seqs / cohort_size)], or nullptr
+  int max_waves;         // the workspace holds partials for this many waves (0 = kMaxDecodeWaves)
   int dtype;
 };
 
@@ -149,14 +150,15 @@ struct DecodeWorkspace {
   size_t shared_slot0;  // first partial slot of the shared phase
   size_t total() const { return cum_bytes + ml_bytes + acc_bytes; }
 };
-inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd, int cohort_size) {
+inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd, int cohort_size,
+                                        int max_waves = kMaxDecodeWaves) {
   const DecodeLayout lay = decode_layout(n_seqs, hn, gn, cohort_size);
   const size_t pairs = (size_t)gn * lay.nsub;
   // one partial per (wave, row, pair) segment: fewer than waves + rows*pairs of them; the shared
   // phase has one per (unit, cohort, pair) segment and wave of the unit
-  const size_t own = (size_t)kMaxDecodeWaves + (size_t)n_seqs * pairs;
+  const size_t own = (size_t)max_waves + (size_t)n_seqs * pairs;
   const size_t shared = lay.n_cohorts > 0
-                            ? (size_t)kMaxDecodeWaves + (((size_t)lay.n_cohorts * pairs) << lay.unit_shift)
+                            ? (size_t)max_waves + (((size_t)lay.n_cohorts * pairs) << lay.unit_shift)
                             : 0;
   const size_t slots = (own + shared) * lay.cols;
   auto pad = [](size_t n) { return (n + 255) & ~(size_t)255; };

@@ -440,7 +440,7 @@ void launch_valu_main(DecodeKP &kp, hipStream_t stream) {
   constexpr int BS = 16;
   constexpr int NW = kDecodeWavesPerWorkgroup;
   int wgs = resident_workgroups<E, HD, GT, BS, NW>();
-  if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
+  if (wgs * NW > kp.max_waves) wgs = kp.max_waves / NW;
   kp.n_waves = wgs * NW;
   hipLaunchKernelGGL((paged_decode_kernel<E, HD, GT, BS, NW>), dim3(wgs), dim3(NW * kWave), 0, stream, kp);
 }
@@ -515,6 +515,7 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.shared_slot0 = a.shared_slot0;
   kp.max_ctx = a.max_context_len;
   kp.n_waves = 0;
+  kp.max_waves = a.max_waves > 0 && a.max_waves < kMaxDecodeWaves ? a.max_waves : kMaxDecodeWaves;
   kp.min_chunk = (a.min_chunk_tokens + 15) / 16;
   kp.tiles_per_block = a.pool.block_size / 16;
   kp.scale_log2e = a.scale * 1.4426950408889634f;

@@ -521,7 +521,7 @@ bool launch_variant(DecodeKP &kp, size_t lds_bytes, hipStream_t stream) {
     seen_bytes = lds_bytes;
   }
   int wgs = per_cu * device_cu_count();
-  if (wgs * NW > kMaxDecodeWaves) wgs = kMaxDecodeWaves / NW;
+  if (wgs * NW > kp.max_waves) wgs = kp.max_waves / NW;
   kp.n_waves = wgs * NW;
   hipLaunchKernelGGL(kernel, dim3(wgs), dim3(NW * kWave), lds_bytes, stream, kp);
   return true;

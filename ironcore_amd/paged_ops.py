@@ -211,6 +211,47 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     return out
 
 
+def paged_decode_static(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                        block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
+                        out: torch.Tensor, scale: float | None = None, min_chunk_tokens: int = 0) -> torch.Tensor:
+    """``paged_decode`` without any allocation: the split-K workspace is the
+    library's own static device array, ``out`` is the caller's.  For callers
+    that may not allocate (graph capture, serving loops).  Batches whose
+    workspace exceeds the array raise ``PagedLibraryError`` (IC_ERR_STATIC_LIMIT);
+    calls that overlap in time on one GPU race on the array."""
+    lib = _lib.load()
+    dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens, out)
+    nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
+    if query.dim() != 3 or query.shape[2] != hd or query.stride(2) != 1 or query.stride(1) != hd:
+        raise ValueError(f"query must be [b, hn, {hd}] with contiguous heads")
+    if query.dtype != k_pool.dtype:
+        raise TypeError("query and pools must share a dtype")
+    b, hn, _ = query.shape
+    if hn % gn != 0:
+        raise ValueError(f"{hn} query heads are not a multiple of {gn} KV heads")
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] != b \
+            or block_tables.stride(1) != 1:
+        raise ValueError("block_tables must be int32 [b, max_blocks] with contiguous rows")
+    if context_lens.dtype != torch.int32 or context_lens.numel() != b or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous int32 [b] tensor")
+    max_context_len = int(max_context_len)
+    if max_context_len > block_tables.shape[1] * bs:
+        raise ValueError("max_context_len exceeds what the block table can address")
+    if out.shape != (b, hn * hd) or out.dtype != query.dtype or out.stride(1) != 1:
+        raise ValueError("out must be [b, hn*hd] in the query dtype with contiguous rows")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    with torch.cuda.device(dev):
+        rc = lib.ic_paged_decode_static(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                        k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                        block_tables.data_ptr(), block_tables.stride(0),
+                                        context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
+                                        float(scale), min_chunk_tokens,
+                                        _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+    _lib.check("ic_paged_decode_static", rc)
+    return out
+
+
 def shared_prefix_blocks(block_tables, context_lens, block_size: int, cohort_size: int):
     """Host-side helper: for each cohort of ``cohort_size`` consecutive rows of
     ``block_tables`` (numpy or CPU tensor, ``[b, max_blocks]``), the number of

@@ -34,7 +34,7 @@ def test_version_and_error_strings():
     lib = _lib.load()
     assert lib.ic_version() >= 100
     assert lib.ic_error_string(0) == b"ok"
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         assert lib.ic_error_string(code) not in (b"", b"unknown error code")
     assert lib.ic_error_string(-99) == b"unknown error code"
 
@@ -118,3 +118,29 @@ def test_python_wrapper_rejects_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU only"):
         paged_ops.kv_append(torch.zeros(1, 1, 64, dtype=torch.bfloat16), torch.zeros(1, 1, 64, dtype=torch.bfloat16),
                             kp, kp, torch.zeros(1, dtype=torch.int64))
+
+
+def _decode_static(**over):
+    a = dict(DECODE_OK, **over)
+    return _lib.load().ic_paged_decode_static(
+        a["out"], a["out_stride"], a["q"], a["q_stride"], a["kp"], a["vp"], a["sb"], a["sh"], a["st"],
+        a["bt"], a["bt_stride"], a["cl"], a["n"], a["hn"], a["gn"], a["hd"], a["bs"], a["nb"],
+        a["max_ctx"], a["scale"], a["chunk"], a["dtype"], None)
+
+
+def test_static_decode_scratch_limit():
+    """The entry point on the library's own scratch refuses, on the host and
+    before anything touches a GPU, a batch whose workspace exceeds the array."""
+    lib = _lib.load()
+    limit = 32 << 20
+    # the BASELINE decode shapes fit
+    for n, hn, gn in [(64, 32, 32), (128, 64, 8), (512, 28, 4)]:
+        need = lib.ic_paged_decode_static_scratch_bytes(n, hn, gn, 128)
+        assert 0 < need <= limit, (n, hn, gn, need)
+        assert need <= lib.ic_paged_decode_workspace_bytes(n, hn, gn, 128)
+    assert lib.ic_paged_decode_static_scratch_bytes(0, 32, 32, 128) == 0
+    assert lib.ic_paged_decode_static_scratch_bytes(4096, 64, 8, 128) > limit
+    assert _decode_static(n=4096, hn=64, gn=8, sb=8 * 16 * 128) == -7
+    assert b"static" in lib.ic_error_string(-7)
+    assert _decode_static(hn=30) == -2
+    assert _decode_static(n=0, q=None, out=None) == 0
