@@ -10,7 +10,9 @@ permuted block tables, q/K/V ~ N(0,1)).  Several layers' pools are resident
 and the steps rotate over them, as a decoder's layers do, so no step re-reads
 bytes the previous one left in cache.
 
-`--workload llama70b | grpo` run the GQA and the shared-prefix decode shapes
+With no `--workload` (or `--workload all`) the other four configurations run
+after the headline one, each under the same gates, and appear in the line's
+`workloads` object.  `--workload llama70b | grpo` run the GQA and the shared-prefix decode shapes
 the same way; `--workload prefill` runs chunked prefill + KV append (16
 sequences, cached prefix uniform in [0, 4096], 512 new tokens each) and
 reports TFLOP/s against the dense bf16 MFMA peak.  `--workload gpt2` runs the
@@ -24,10 +26,13 @@ beside it.
 Prints ONE JSON line.  For decode `value` is achieved HBM GB/s of the whole
 step (algorithmic bytes / wall time per step), with decode tokens/s beside it;
 `roofline` describes the dominant call (decode: main kernel + its split-K
-reduce; prefill: the MFMA kernel) timed with events on the launch stream;
-`cpu_baseline` is the CPU oracle (the reference's dense attention arithmetic
-driven through the block table) timed on the host cores on a bounded sample
-of the same workload.
+reduce; prefill: the MFMA kernel) timed with events on the launch stream in a
+pass of its own after the wall-timed steps (EVENT_LAUNCHES launches, each
+bracketed by an event pair); `cpu_baseline` is the CPU oracle (the
+reference's dense attention arithmetic driven through the block table) timed
+on the host cores on the same workload.  Before anything is timed every
+sequence of the batch is checked against the oracle (max-abs 2e-2, bf16) and
+the appended rows are compared with the pool bit for bit.
 """
 from __future__ import annotations
 
@@ -41,10 +46,31 @@ import time
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
 
-# HBM bytes per launch of the decode main kernel (workload, seed 0), from
-# FETCH_SIZE / WRITE_SIZE counter runs scaled by a 1 GiB device copy in the
-# same process (the counter summaries under profiles/ hold the raw figures).
-MEASURED_TRAFFIC = {("llama7b", 0): 2465266534, ("llama70b", 0): 2479865549, ("grpo", 0): 677594009}
+EVENT_LAUNCHES = 40         # event-bracketed launches of the dominant call behind `roofline`
+PARITY_BAR = 2e-2           # max-abs against the oracle, bf16 (the bar the target states)
+ROOT = os.path.dirname(os.path.abspath(__file__))
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(workload, seed):
+    """HBM bytes per launch of the workload's dominant kernel as the profiler's
+    FETCH_SIZE / WRITE_SIZE counters gave them (profiles/traffic.json holds
+    the counter readings, the scale factors from a copy of known size and a
+    digest of the kernel sources they were measured on).  A figure measured
+    on other sources than the ones that are about to run is not reported:
+    returns (bytes or None, stale flag)."""
+    from ironcore_amd import build as ic_build
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, False
+    ent = rec.get("workloads", {}).get(workload)
+    if ent is None or ent.get("seed", 0) != seed:
+        return None, False
+    if rec.get("csrc_sha256") != ic_build.csrc_digest():
+        return None, True
+    return int(ent["hbm_bytes_per_launch"]), False
 
 
 def parse():
@@ -54,19 +80,23 @@ def parse():
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default 20; gpt2: 1)")
     ap.add_argument("--layers", type=int, default=4, help="resident layer pools the steps rotate over")
     ap.add_argument("--min-chunk-tokens", type=int, default=0, help="smallest split-K share (0 = library default)")
-    ap.add_argument("--workload", default="llama7b", choices=["llama7b", "llama70b", "grpo", "prefill", "gpt2"])
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "llama7b", "llama70b", "grpo", "prefill", "gpt2"],
+                    help="all = the headline line (llama7b) with the other four configurations under `workloads`")
     ap.add_argument("--cohort-size", type=int, default=0,
                     help="shared-prefix cohort size for decode (0 = the samples per prompt of the workload, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline time budget")
+    ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU baseline time budget per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so a counter run can be scaled")
     args = ap.parse_args()
+    args.gpt2_steps = args.steps if args.workload == "gpt2" and args.steps else 5
+    args.gpt2_warmup = args.warmup if args.workload == "gpt2" and args.warmup is not None else 1
     if args.steps is None:
-        args.steps = 5 if args.workload == "gpt2" else 200
+        args.steps = 200
     if args.warmup is None:
-        args.warmup = 1 if args.workload == "gpt2" else 20
+        args.warmup = 20
     return args
 
 
@@ -87,34 +117,48 @@ def copy_calibration(torch, dev):
     torch.cuda.synchronize()
 
 
-EVENT_EVERY = 8   # steps between event pairs: recording costs launch slots of its own
-
-
-def time_steps(torch, step, steps, warmup):
+def time_steps(torch, step, steps, warmup, event_launches=EVENT_LAUNCHES):
     """Run `warmup` untimed steps, then exactly `steps` timed ones bracketed by
-    synchronisations.  `step(i, ev)` enqueues step i and, when `ev` is not None,
-    records the event pair `ev` around its dominant call; every EVENT_EVERY-th
-    timed step is sampled that way (an event pair per step would add two launch
-    slots to each step of the region being timed).  Returns (ms per step by
-    wall clock, list of per-call ms from the events)."""
+    synchronisations (no events inside: an event pair costs a step two launch
+    slots), then a pass of `event_launches` further steps each of which
+    records an event pair around its dominant call.  `step(i, ev)` enqueues
+    step i and records `ev` when it is not None.  Returns (ms per step by wall
+    clock, list of per-call ms from the events)."""
     for i in range(warmup):
         step(i, None)
     torch.cuda.synchronize()
-    ev = {i: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for i in range(0, steps, EVENT_EVERY)}
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i, ev.get(i))
+        step(i, None)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in ev.values()]
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(event_launches)]
+    for i, pair in enumerate(ev):
+        step(steps + i, pair)
+    torch.cuda.synchronize()
+    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in ev]
 
 
-def bench_decode(args, torch, dev):
+def timed_oracle(fn, budget_s):
+    """The parity gate's oracle call doubles as the CPU baseline: run it once
+    (result kept for the gate), then again while the budget lasts (at most two
+    more), and report the median.  Returns (result, seconds, runs)."""
+    t0 = time.perf_counter()
+    ref = fn()
+    times = [time.perf_counter() - t0]
+    while len(times) < 3 and sum(times) + times[-1] <= budget_s:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return ref, statistics.median(times), len(times)
+
+
+def bench_decode(args, torch, dev, workload):
     from ironcore_amd import paged_ops, workloads
     from oracle import paged as oracle_paged
     make = {"llama7b": workloads.llama7b_decode, "llama70b": workloads.llama70b_gqa_decode,
-            "grpo": workloads.qwen7b_grpo_decode}[args.workload]
+            "grpo": workloads.qwen7b_grpo_decode}[workload]
     wl = make(device=dev, seed=args.seed)
     b, hn, gn, hd, bs = wl.batch, wl.hn, wl.gn, wl.hd, wl.block_size
     pools = [(wl.k_pool, wl.v_pool)]          # one pool pair per resident layer
@@ -151,15 +195,24 @@ def bench_decode(args, torch, dev):
         if ev:
             ev[1].record()
 
-    # parity gate on the tensors that are about to be timed
+    # parity gate on the tensors that are about to be timed: EVERY sequence of the batch against
+    # the oracle, and the appended rows against the pool bit for bit
     step(0, None)
     torch.cuda.synchronize()
-    n_chk = min(b, 6)
-    ref = oracle_paged.paged_decode(wl.query[:n_chk].cpu(), pools[0][0].cpu(), pools[0][1].cpu(),
-                                    wl.block_tables[:n_chk].cpu(), wl.context_lens[:n_chk].cpu())
-    parity = (out[:n_chk].float().cpu() - ref.float()).abs().max().item()
-    if not parity <= 2e-2:
-        sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
+    kp_cpu, vp_cpu = pools[0][0].cpu(), pools[0][1].cpu()
+    q_cpu, bt_cpu, cl_cpu = wl.query.cpu(), wl.block_tables.cpu(), wl.context_lens.cpu()
+    ref, cpu_s, cpu_runs = timed_oracle(
+        lambda: oracle_paged.paged_decode(q_cpu, kp_cpu, vp_cpu, bt_cpu, cl_cpu),
+        0.0 if args.no_cpu_baseline else args.cpu_seconds)
+    parity = (out.float().cpu() - ref.float()).abs().max().item()
+    if not parity <= PARITY_BAR:
+        sys.exit(f"parity gate failed ({wl.name}): max|out - oracle| = {parity} > {PARITY_BAR}")
+    sm = slot_mapping.cpu()
+    for pool_cpu, new in ((kp_cpu, k_new), (vp_cpu, v_new)):
+        got = pool_cpu[sm // bs, :, sm % bs, :]
+        if not torch.equal(got.view(torch.int16), new.cpu().view(torch.int16)):
+            sys.exit(f"parity gate failed ({wl.name}): appended rows differ from the pool")
+    del kp_cpu, vp_cpu, ref
     if args.copy_calibration:
         copy_calibration(torch, dev)
 
@@ -170,6 +223,7 @@ def bench_decode(args, torch, dev):
     append_bytes = 2 * (2 * b * gn * hd * es) + 8 * b
     value = (decode_bytes + append_bytes) / (ms_per_step * 1e-3) / 1e9
     achieved = decode_bytes / (decode_ms_avg * 1e-3) / 1e9
+    traffic, stale = measured_traffic(workload, args.seed)
     result = {
         "metric": "paged_decode_hbm_gbps", "value": round(value, 1), "unit": "GB/s",
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
@@ -185,41 +239,25 @@ def bench_decode(args, torch, dev):
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.seed)),
+                     "traffic": traffic,
                      "kernel": "paged_decode_mfma_kernel (+ paged_decode_reduce_kernel)",
                      "bytes_per_launch": decode_bytes, "avg_launch_ms": round(decode_ms_avg, 5),
-                     "median_launch_ms": round(statistics.median(decode_ms), 5)},
+                     "median_launch_ms": round(statistics.median(decode_ms), 5),
+                     "n_event_samples": len(decode_ms)},
     }
+    if stale:
+        result["roofline"]["traffic_stale"] = True
     if wl.logical_tokens != wl.unique_tokens:
         logical = wl.logical_tokens * wl.kv_bytes_per_token()
         result["logical_kv_gbps"] = round(logical / (decode_ms_avg * 1e-3) / 1e9, 1)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline_decode(wl, pools[0], args.cpu_seconds)
+        tokens = wl.logical_tokens
+        result["cpu_baseline"] = {
+            "value": round(tokens * wl.kv_bytes_per_token() / cpu_s / 1e9, 3), "unit": "GB/s", "kind": "port",
+            "sample": f"all {b} sequences of the same batch, one layer, median of {cpu_runs} run(s) of the "
+                      f"oracle (gather through the block table + dense attention); {tokens} context tokens",
+            "tokens_per_s_per_layer": round(b / cpu_s, 2), **cpu_info()}
     return result
-
-
-def cpu_baseline_decode(wl, pool, budget_s):
-    """The CPU oracle on a bounded sample: the first n sequences of the same
-    batch (same block tables, same pools), median of 3 repetitions."""
-    from oracle import paged as oracle_paged
-    kp, vp = pool[0].cpu(), pool[1].cpu()
-    q, bt, cl = wl.query.cpu(), wl.block_tables.cpu(), wl.context_lens.cpu()
-    n = min(wl.batch, 8)
-    t0 = time.perf_counter()
-    oracle_paged.paged_decode(q[:n], kp, vp, bt[:n], cl[:n])       # warm-up, also sizes the sample
-    per_seq = (time.perf_counter() - t0) / n
-    n = int(max(1, min(wl.batch, budget_s / 4 / max(per_seq, 1e-6))))
-    times = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        oracle_paged.paged_decode(q[:n], kp, vp, bt[:n], cl[:n])
-        times.append(time.perf_counter() - t0)
-    t = statistics.median(times)
-    tokens = int(cl[:n].sum())
-    return {"value": round(tokens * wl.kv_bytes_per_token() / t / 1e9, 3), "unit": "GB/s", "kind": "port",
-            "sample": f"first {n} of {wl.batch} sequences of the same batch, one layer, "
-                      f"median of 3 (after 1 warm-up); {tokens} context tokens",
-            "tokens_per_s_per_layer": round(n / t, 2), **cpu_info()}
 
 
 def bench_prefill(args, torch, dev):
@@ -237,17 +275,23 @@ def bench_prefill(args, torch, dev):
         if ev:
             ev[1].record()
 
-    # parity gate: the sequence with the shortest prefix, all heads, against the oracle
+    # parity gate: ALL sequences, all heads, against the oracle; the appended rows against the
+    # pool bit for bit
     step(0, None)
     torch.cuda.synchronize()
-    i = min(range(len(wl.prefix_lens)), key=lambda j: wl.prefix_lens[j])
-    lo, hi = int(wl.cu_seqlens_q[i]), int(wl.cu_seqlens_q[i + 1])
-    one = (wl.query[lo:hi].cpu(), wl.k_pool.cpu(), wl.v_pool.cpu(), wl.block_tables[i:i + 1].cpu(),
-           wl.context_lens[i:i + 1].cpu(), torch.tensor([0, hi - lo], dtype=torch.int32))
-    ref = oracle_paged.paged_prefill(*one)
-    parity = (out[lo:hi].float().cpu() - ref.float()).abs().max().item()
-    if not parity <= 2e-2:
-        sys.exit(f"parity gate failed: max|out - oracle| = {parity} > 2e-2")
+    cpu = (wl.query.cpu(), wl.k_pool.cpu(), wl.v_pool.cpu(), wl.block_tables.cpu(), wl.context_lens.cpu(),
+           wl.cu_seqlens_q.cpu())
+    ref, cpu_s, cpu_runs = timed_oracle(lambda: oracle_paged.paged_prefill(*cpu),
+                                        0.0 if args.no_cpu_baseline else args.cpu_seconds)
+    parity = (out.float().cpu() - ref.float()).abs().max().item()
+    if not parity <= PARITY_BAR:
+        sys.exit(f"parity gate failed ({wl.name}): max|out - oracle| = {parity} > {PARITY_BAR}")
+    sm = wl.slot_mapping.cpu()
+    for pool_cpu, new in ((cpu[1], wl.k_new), (cpu[2], wl.v_new)):
+        got = pool_cpu[sm // wl.block_size, :, sm % wl.block_size, :]
+        if not torch.equal(got.view(torch.int16), new.cpu().view(torch.int16)):
+            sys.exit(f"parity gate failed ({wl.name}): appended rows differ from the pool")
+    del cpu, ref
     if args.copy_calibration:
         copy_calibration(torch, dev)
 
@@ -258,6 +302,7 @@ def bench_prefill(args, torch, dev):
     append_bytes = 2 * 2 * wl.k_new.numel() * es
     tflops = flops / (call_avg * 1e-3) / 1e12
     n_tok = wl.query.shape[0]
+    traffic, stale = measured_traffic("prefill", args.seed)
 
     def append_only(i, ev):
         if ev:
@@ -265,12 +310,13 @@ def bench_prefill(args, torch, dev):
         paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)
         if ev:
             ev[1].record()
-    _, app_ms = time_steps(torch, append_only, 50, 5)
+    _, app_ms = time_steps(torch, append_only, 5, 5)
 
     # the same append with rotary embedding fused in (Q rotated in place, K rotated
     # into the pool, V copied), timed the same way on a scratch copy of the query
-    from oracle import rope as oracle_rope
-    cos_t, sin_t = (t.to(dev) for t in oracle_rope.rope_tables(wl.hd, 8192))
+    from ironcore_amd.layers.rotary import RotaryPositionalEmbedding
+    rope = RotaryPositionalEmbedding(wl.hd, max_seq_len=8192).to(dev)
+    cos_t, sin_t = rope.cos_emb, rope.sin_emb
     q_rot = wl.query.clone()
     pos = torch.cat([torch.arange(pf, pf + c, dtype=torch.int32) for pf, c in zip(wl.prefix_lens, wl.chunk_lens)]
                     ).to(dev)
@@ -282,7 +328,7 @@ def bench_prefill(args, torch, dev):
                                  cos_t, sin_t)
         if ev:
             ev[1].record()
-    _, rope_ms = time_steps(torch, rope_append_only, 50, 5)
+    _, rope_ms = time_steps(torch, rope_append_only, 5, 5)
     rope_bytes = append_bytes + 2 * wl.query.numel() * es
     paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)  # leave the pool unrotated
 
@@ -300,18 +346,18 @@ def bench_prefill(args, torch, dev):
         "append_hbm_gbps": round(append_bytes / (statistics.mean(app_ms) * 1e-3) / 1e9, 1),
         "rope_append_hbm_gbps": round(rope_bytes / (statistics.mean(rope_ms) * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
                      "kernel": "paged_prefill_kernel", "flops_per_launch": flops,
-                     "avg_launch_ms": round(call_avg, 5), "median_launch_ms": round(statistics.median(call_ms), 5)},
+                     "avg_launch_ms": round(call_avg, 5), "median_launch_ms": round(statistics.median(call_ms), 5),
+                     "n_event_samples": len(call_ms)},
     }
+    if stale:
+        result["roofline"]["traffic_stale"] = True
     if not args.no_cpu_baseline:
-        t0 = time.perf_counter()
-        oracle_paged.paged_prefill(*one)
-        t = time.perf_counter() - t0
-        c, pfx = wl.chunk_lens[i], wl.prefix_lens[i]
-        f = 4 * wl.hn * wl.hd * (c * pfx + c * (c + 1) // 2)
-        result["cpu_baseline"] = {"value": round(f / t / 1e12, 4), "unit": "TFLOP/s", "kind": "port",
-                                  "sample": f"one sequence of the batch (prefix {pfx}, chunk {c}), all heads, 1 run",
+        result["cpu_baseline"] = {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "kind": "port",
+                                  "sample": f"all {len(wl.chunk_lens)} sequences of the batch, all heads, median of "
+                                            f"{cpu_runs} run(s) of the oracle (gather through the block table + dense "
+                                            "attention under the shifted causal mask)",
                                   **cpu_info()}
     return result
 
@@ -343,14 +389,14 @@ def bench_gpt2(args, torch, dev):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps, out
 
-    sec, got = timed(lambda: generation.generate(model, ids_dev, new, use_graph=True), args.steps, args.warmup)
-    sec_eager, got_eager = timed(lambda: generation.generate(model, ids_dev, new), args.steps, args.warmup)
+    sec, got = timed(lambda: generation.generate(model, ids_dev, new, use_graph=True), args.gpt2_steps, args.gpt2_warmup)
+    sec_eager, got_eager = timed(lambda: generation.generate(model, ids_dev, new), args.gpt2_steps, args.gpt2_warmup)
     sec_full, got_full = timed(lambda: generation.generate_full_recompute(model, ids_dev, new), 1, 0)
     if not torch.equal(got, got_eager):
         sys.exit("parity gate failed: the graph-replay loop and the step-by-step loop chose different tokens")
     result = {
         "metric": "generate_tokens_per_s", "value": round(batch * new / sec, 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3),
+        "n_gpus": 1, "steps": args.gpt2_steps, "warmup": args.gpt2_warmup, "ms_per_step": round(sec * 1e3, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gpt2-small end to end: random-init fp32, batch 4, prompt 128, greedy 64 new tokens, "
                                "block 16",
@@ -391,8 +437,35 @@ def main():
         sys.exit("bench.py needs a GPU (the paged path has no CPU implementation)")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    run = {"prefill": bench_prefill, "gpt2": bench_gpt2}.get(args.workload, bench_decode)
-    result = run(args, torch, dev)
+    def run(workload):
+        if workload == "prefill":
+            res = bench_prefill(args, torch, dev)
+        elif workload == "gpt2":
+            res = bench_gpt2(args, torch, dev)
+        else:
+            res = bench_decode(args, torch, dev, workload)
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()  # the next workload's pools take the place of this one's
+        return res
+
+    if args.workload != "all":
+        print(json.dumps(run(args.workload)))
+        return
+    t0 = time.perf_counter()
+    result = run("llama7b")
+    # the other configurations, each gated and measured the same way; an entry keeps the fields
+    # that describe a measurement and drops the ones that repeat the top-level line's
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype", "config", "roofline",
+            "cpu_baseline", "parity_max_abs_vs_oracle", "pct_of_hbm_peak", "decode_tokens_per_s_per_layer",
+            "logical_kv_gbps", "prefill_tokens_per_s_per_layer", "append_hbm_gbps", "rope_append_hbm_gbps",
+            "tokens_identical_to_oracle", "step_by_step_tokens_per_s_gpu", "full_recompute_tokens_per_s_gpu",
+            "paged_equals_full_recompute_gpu", "min_top1_top2_margin")
+    result["workloads"] = {"llama7b": {k: result[k] for k in keep if k in result}}
+    for w in ("llama70b", "grpo", "prefill", "gpt2"):
+        r = run(w)
+        result["workloads"][w] = {k: r[k] for k in keep if k in r}
+    result["bench_wall_s"] = round(time.perf_counter() - t0, 1)
     print(json.dumps(result))
 
 

@@ -272,6 +272,61 @@ int ic_paged_prefill(void *out, int64_t out_stride_token,
                      int64_t num_blocks, float scale, int causal,
                      int dtype, void *stream);
 
+/*
+ * Chunked prefill under a general attention mask: ic_paged_prefill with the
+ * causal rule replaced by the caller's mask, for the attention_mask argument
+ * of ironcore/layers/attention.py:208-253 when it is neither absent nor the
+ * causal pattern (any mask broadcastable to [b, 1, sq, sk], attention.py:115-117;
+ * e.g. the per-document masks of ironcore/language_model.py:140-152).
+ *
+ *   mask    uint8; the byte of (sequence i, query head h, chunk row r, key j) is
+ *           mask[i*mask_stride_seq + h*mask_stride_head + r*mask_stride_row + j],
+ *           nonzero = visible.  A stride of 0 broadcasts over that index.  Rows
+ *           must cover context_lens[i] keys.
+ * Hidden keys get the reference's FINITE fill value (attention.py:66): next to a
+ * visible key they weigh nothing; a query row with no visible key returns the
+ * plain average of V over its context, as the reference does.  A chunk may be
+ * longer than its context here (sq > sk).  bf16 / fp16 only.
+ */
+int ic_paged_prefill_masked(void *out, int64_t out_stride_token,
+                            const void *q, int64_t q_stride_token,
+                            const void *k_pool, const void *v_pool,
+                            int64_t pool_stride_block, int64_t pool_stride_head,
+                            int64_t pool_stride_token,
+                            const int32_t *block_tables, int64_t block_table_stride,
+                            const int32_t *context_lens, const int32_t *cu_seqlens_q,
+                            int n_seqs, int max_chunk_len,
+                            int hn, int gn, int hd, int block_size,
+                            int64_t num_blocks, float scale,
+                            const uint8_t *mask, int64_t mask_stride_seq,
+                            int64_t mask_stride_head, int64_t mask_stride_row,
+                            int dtype, void *stream);
+
+/*
+ * Paged decode under a key mask, fp32 only: ic_paged_decode where sequence i's
+ * query head h sees key j only if
+ * key_mask[i*key_mask_stride_seq + h*key_mask_stride_head + j] is nonzero
+ * (key_mask_stride_head 0 = one mask row for all heads; key_mask_stride_seq
+ * >= max_context_len).  Same finite-fill semantics as ic_paged_prefill_masked.
+ * It is how an fp32 attention call with a general mask runs (one decode row
+ * per query row; fp32 has no matrix-core path); 16-bit calls use
+ * ic_paged_prefill_masked and get IC_ERR_UNSUPPORTED here.
+ */
+int ic_paged_decode_masked(void *out, int64_t out_stride_seq,
+                           const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool,
+                           int64_t pool_stride_block, int64_t pool_stride_head,
+                           int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens,
+                           int n_seqs, int hn, int gn, int hd, int block_size,
+                           int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens,
+                           const uint8_t *key_mask, int64_t key_mask_stride_seq,
+                           int64_t key_mask_stride_head,
+                           void *workspace, size_t workspace_bytes,
+                           int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

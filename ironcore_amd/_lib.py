@@ -76,6 +76,27 @@ SIGNATURES = {
         c_int, c_int, c_int, c_int,             # hn, gn, hd, block_size
         c_int64, c_float, c_int,                # num_blocks, scale, causal
         c_int, c_void_p]),                      # dtype, stream
+    "ic_paged_prefill_masked": (c_int, [
+        c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
+        c_void_p, c_void_p,                     # k_pool, v_pool
+        c_int64, c_int64, c_int64,              # pool strides
+        c_void_p, c_int64, c_void_p, c_void_p,  # block_tables, stride, context_lens, cu_seqlens_q
+        c_int, c_int,                           # n_seqs, max_chunk_len
+        c_int, c_int, c_int, c_int,             # hn, gn, hd, block_size
+        c_int64, c_float,                       # num_blocks, scale
+        c_void_p, c_int64, c_int64, c_int64,    # mask, strides: seq, head, row
+        c_int, c_void_p]),                      # dtype, stream
+    "ic_paged_decode_masked": (c_int, [
+        c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
+        c_void_p, c_void_p,                     # k_pool, v_pool
+        c_int64, c_int64, c_int64,              # pool strides
+        c_void_p, c_int64, c_void_p,            # block_tables, stride, context_lens
+        c_int, c_int, c_int, c_int, c_int,      # n_seqs, hn, gn, hd, block_size
+        c_int64, c_int, c_float,                # num_blocks, max_context_len, scale
+        c_int,                                  # min_chunk_tokens
+        c_void_p, c_int64, c_int64,             # key_mask, strides: seq, head
+        c_void_p, c_size_t,                     # workspace, workspace_bytes
+        c_int, c_void_p]),                      # dtype, stream
 }
 
 

@@ -35,6 +35,20 @@ HIPCC_FLAGS = [
 ]
 
 
+def csrc_digest() -> str:
+    """SHA-256 over the names and contents of the kernel sources (csrc/*.hip,
+    *.h): identifies the code a profiler figure was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(CSRC.glob("*")):
+        if path.suffix in (".hip", ".h"):
+            h.update(path.name.encode())
+            h.update(b"\0")
+            h.update(path.read_bytes())
+            h.update(b"\0")
+    return h.hexdigest()
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):

@@ -57,9 +57,19 @@ struct DecodeKP {
   int n_cohorts;
   int spw;
   int unit_shift;
+  // Key mask (vector-ALU kernel only; nullptr = every key of the context is visible): byte
+  // (sequence i, query head h, key j) at key_mask[i*key_mask_stride_seq + h*key_mask_stride_head + j],
+  // nonzero = visible.
+  const uint8_t *key_mask;
+  int64_t key_mask_stride_seq;
+  int64_t key_mask_stride_head;
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
+// Score (log2 units) of a key the mask hides: the reference fills hidden scores with the FINITE
+// minimum of the element type (attention.py:66,115-117), so beside a visible key a hidden one
+// weighs nothing, while a row with no visible key averages V over its whole context.
+constexpr float kHiddenLog2 = -0x1p100f;
 
 __device__ __forceinline__ int seq_blocks(const DecodeKP &p, int seq, int bs) {
   int ctx = p.context_lens[seq];

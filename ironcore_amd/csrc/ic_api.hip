@@ -64,9 +64,15 @@ int decode_checked(void *out, int64_t out_stride_seq, const void *q, int64_t q_s
                    int64_t block_table_stride, const int32_t *context_lens, int n_seqs, int hn, int gn,
                    int hd, int block_size, int64_t num_blocks, int max_context_len, float scale,
                    int min_chunk_tokens, int cohort_size, const int32_t *cohort_shared_blocks,
-                   void *workspace, size_t workspace_bytes, int max_waves, int dtype, void *stream) {
+                   void *workspace, size_t workspace_bytes, int max_waves, int dtype, void *stream,
+                   const uint8_t *key_mask = nullptr, int64_t key_mask_stride_seq = 0,
+                   int64_t key_mask_stride_head = 0) {
   if (n_seqs < 0 || hn <= 0 || gn <= 0 || hn % gn != 0 || max_context_len < 0 || cohort_size < 1)
     return IC_ERR_BAD_SHAPE;
+  if (key_mask != nullptr) {
+    if (dtype != IC_DTYPE_F32 || cohort_size != 1) return IC_ERR_UNSUPPORTED;
+    if (key_mask_stride_seq < max_context_len || key_mask_stride_head < 0) return IC_ERR_BAD_SHAPE;
+  }
   if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
   const int es = ic::elem_size(dtype);
   if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
@@ -118,8 +124,60 @@ int decode_checked(void *out, int64_t out_stride_seq, const void *q, int64_t q_s
   a.cohort_size = cohort_size;
   a.cohort_shared_blocks = cohort_shared_blocks;
   a.max_waves = max_waves;
+  a.key_mask = key_mask;
+  a.key_mask_stride_seq = key_mask_stride_seq;
+  a.key_mask_stride_head = key_mask_stride_head;
   a.dtype = dtype;
   return ic::launch_paged_decode(a, static_cast<hipStream_t>(stream));
+}
+
+int prefill_checked(void *out, int64_t out_stride_token, const void *q, int64_t q_stride_token,
+                    const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                    int64_t pool_stride_head, int64_t pool_stride_token, const int32_t *block_tables,
+                    int64_t block_table_stride, const int32_t *context_lens, const int32_t *cu_seqlens_q,
+                    int n_seqs, int max_chunk_len, int hn, int gn, int hd, int block_size,
+                    int64_t num_blocks, float scale, int causal, const uint8_t *mask,
+                    int64_t mask_stride_seq, int64_t mask_stride_head, int64_t mask_stride_row, int dtype,
+                    void *stream) {
+  if (n_seqs < 0 || max_chunk_len < 0 || hn <= 0 || gn <= 0 || hn % gn != 0) return IC_ERR_BAD_SHAPE;
+  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
+  const int es = ic::elem_size(dtype);
+  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
+                          num_blocks, es))
+    return rc;
+  if (n_seqs == 0 || max_chunk_len == 0) return IC_OK;
+  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens || !cu_seqlens_q)
+    return IC_ERR_NULL_POINTER;
+  if (out_stride_token < (int64_t)hn * hd || q_stride_token < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
+  if (block_table_stride <= 0) return IC_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(out) || !aligned16(k_pool) || !aligned16(v_pool) ||
+      !stride16(q_stride_token, es) || !stride16(out_stride_token, es))
+    return IC_ERR_ALIGNMENT;
+  ic::PrefillArgs a;
+  a.out = out;
+  a.out_stride_token = out_stride_token;
+  a.q = q;
+  a.q_stride_token = q_stride_token;
+  a.k_pool = k_pool;
+  a.v_pool = v_pool;
+  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
+  a.block_tables = block_tables;
+  a.block_table_stride = block_table_stride;
+  a.context_lens = context_lens;
+  a.cu_seqlens_q = cu_seqlens_q;
+  a.n_seqs = n_seqs;
+  a.max_chunk_len = max_chunk_len;
+  a.hn = hn;
+  a.gn = gn;
+  a.hd = hd;
+  a.scale = scale;
+  a.causal = causal;
+  a.dtype = dtype;
+  a.mask = mask;
+  a.mask_stride_seq = mask_stride_seq;
+  a.mask_stride_head = mask_stride_head;
+  a.mask_stride_row = mask_stride_row;
+  return ic::launch_paged_prefill(a, static_cast<hipStream_t>(stream));
 }
 
 }  // namespace
@@ -322,41 +380,46 @@ int ic_paged_prefill(void *out, int64_t out_stride_token, const void *q, int64_t
                      const int32_t *context_lens, const int32_t *cu_seqlens_q, int n_seqs,
                      int max_chunk_len, int hn, int gn, int hd, int block_size, int64_t num_blocks,
                      float scale, int causal, int dtype, void *stream) {
-  if (n_seqs < 0 || max_chunk_len < 0 || hn <= 0 || gn <= 0 || hn % gn != 0) return IC_ERR_BAD_SHAPE;
-  if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
-  const int es = ic::elem_size(dtype);
-  if (int rc = check_pool(pool_stride_block, pool_stride_head, pool_stride_token, gn, hd, block_size,
-                          num_blocks, es))
-    return rc;
-  if (n_seqs == 0 || max_chunk_len == 0) return IC_OK;
-  if (!out || !q || !k_pool || !v_pool || !block_tables || !context_lens || !cu_seqlens_q)
-    return IC_ERR_NULL_POINTER;
-  if (out_stride_token < (int64_t)hn * hd || q_stride_token < (int64_t)hn * hd) return IC_ERR_BAD_SHAPE;
-  if (block_table_stride <= 0) return IC_ERR_BAD_SHAPE;
-  if (!aligned16(q) || !aligned16(out) || !aligned16(k_pool) || !aligned16(v_pool) ||
-      !stride16(q_stride_token, es) || !stride16(out_stride_token, es))
-    return IC_ERR_ALIGNMENT;
-  ic::PrefillArgs a;
-  a.out = out;
-  a.out_stride_token = out_stride_token;
-  a.q = q;
-  a.q_stride_token = q_stride_token;
-  a.k_pool = k_pool;
-  a.v_pool = v_pool;
-  a.pool = {pool_stride_block, pool_stride_head, pool_stride_token, num_blocks, block_size};
-  a.block_tables = block_tables;
-  a.block_table_stride = block_table_stride;
-  a.context_lens = context_lens;
-  a.cu_seqlens_q = cu_seqlens_q;
-  a.n_seqs = n_seqs;
-  a.max_chunk_len = max_chunk_len;
-  a.hn = hn;
-  a.gn = gn;
-  a.hd = hd;
-  a.scale = scale;
-  a.causal = causal;
-  a.dtype = dtype;
-  return ic::launch_paged_prefill(a, static_cast<hipStream_t>(stream));
+  return prefill_checked(out, out_stride_token, q, q_stride_token, k_pool, v_pool, pool_stride_block,
+                         pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                         context_lens, cu_seqlens_q, n_seqs, max_chunk_len, hn, gn, hd, block_size,
+                         num_blocks, scale, causal, nullptr, 0, 0, 0, dtype, stream);
+}
+
+int ic_paged_prefill_masked(void *out, int64_t out_stride_token, const void *q, int64_t q_stride_token,
+                            const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                            int64_t pool_stride_head, int64_t pool_stride_token,
+                            const int32_t *block_tables, int64_t block_table_stride,
+                            const int32_t *context_lens, const int32_t *cu_seqlens_q, int n_seqs,
+                            int max_chunk_len, int hn, int gn, int hd, int block_size,
+                            int64_t num_blocks, float scale, const uint8_t *mask,
+                            int64_t mask_stride_seq, int64_t mask_stride_head, int64_t mask_stride_row,
+                            int dtype, void *stream) {
+  if (n_seqs > 0 && max_chunk_len > 0 && mask == nullptr) return IC_ERR_NULL_POINTER;
+  if (mask_stride_seq < 0 || mask_stride_head < 0 || mask_stride_row < 0) return IC_ERR_BAD_SHAPE;
+  return prefill_checked(out, out_stride_token, q, q_stride_token, k_pool, v_pool, pool_stride_block,
+                         pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                         context_lens, cu_seqlens_q, n_seqs, max_chunk_len, hn, gn, hd, block_size,
+                         num_blocks, scale, 0, mask, mask_stride_seq, mask_stride_head, mask_stride_row,
+                         dtype, stream);
+}
+
+int ic_paged_decode_masked(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,
+                           const void *k_pool, const void *v_pool, int64_t pool_stride_block,
+                           int64_t pool_stride_head, int64_t pool_stride_token,
+                           const int32_t *block_tables, int64_t block_table_stride,
+                           const int32_t *context_lens, int n_seqs, int hn, int gn, int hd,
+                           int block_size, int64_t num_blocks, int max_context_len, float scale,
+                           int min_chunk_tokens, const uint8_t *key_mask, int64_t key_mask_stride_seq,
+                           int64_t key_mask_stride_head, void *workspace, size_t workspace_bytes,
+                           int dtype, void *stream) {
+  if (n_seqs > 0 && key_mask == nullptr) return IC_ERR_NULL_POINTER;
+  return decode_checked(out, out_stride_seq, q, q_stride_seq, k_pool, v_pool, pool_stride_block,
+                        pool_stride_head, pool_stride_token, block_tables, block_table_stride,
+                        context_lens, n_seqs, hn, gn, hd, block_size, num_blocks, max_context_len,
+                        scale, min_chunk_tokens, 1, nullptr, workspace, workspace_bytes,
+                        ic::kMaxDecodeWaves, dtype, stream, key_mask, key_mask_stride_seq,
+                        key_mask_stride_head);
 }
 
 }  // extern "C"

@@ -69,6 +69,11 @@ struct DecodeArgs {
   const int32_t *cohort_shared_blocks;  // [ceil(n_seqs / cohort_size)], or nullptr
   int max_waves;         // the workspace holds partials for this many waves (0 = kMaxDecodeWaves)
   int dtype;
+  // optional key mask (fp32 kernel only): byte (sequence, query head, key) at
+  // seq*key_mask_stride_seq + head*key_mask_stride_head + key, nonzero = visible
+  const uint8_t *key_mask = nullptr;
+  int64_t key_mask_stride_seq = 0;
+  int64_t key_mask_stride_head = 0;
 };
 
 struct PrefillArgs {
@@ -91,6 +96,12 @@ struct PrefillArgs {
   float scale;
   int causal;
   int dtype;
+  // optional byte mask (nullptr = the causal rule / no mask): element (sequence, head, chunk row,
+  // key) at seq*mask_stride_seq + head*mask_stride_head + row*mask_stride_row + key
+  const uint8_t *mask = nullptr;
+  int64_t mask_stride_seq = 0;
+  int64_t mask_stride_head = 0;
+  int64_t mask_stride_row = 0;
 };
 
 // Each returns IC_OK, IC_ERR_UNSUPPORTED (no kernel built for this

@@ -212,6 +212,23 @@ __global__ __launch_bounds__(NW *kWave) void paged_decode_kernel(const DecodeKP 
         }
       }
     }
+    if (p.key_mask != nullptr) {  // keys the caller's mask hides (context-length cuts stay -inf)
+      int ctx = p.context_lens[c.seq];
+      ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
+      const int kvh = c.pair / p.nsub;
+      const int head0 = kvh * p.group + (c.pair - kvh * p.nsub) * GT;
+      const uint8_t *mrow = p.key_mask + c.seq * p.key_mask_stride_seq + c.blk * BS + rowg;
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        if (c.blk * BS + i * RPL + rowg < ctx) {
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            const int h = head0 + g < p.hn ? head0 + g : p.hn - 1;
+            if (mrow[h * p.key_mask_stride_head + i * RPL] == 0) s[g][i] = kHiddenLog2;
+          }
+        }
+      }
+    }
     float vf[NLD][EPL];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) E::widen(vv[i], vf[i]);
@@ -519,6 +536,10 @@ int launch_paged_decode(const DecodeArgs &a, hipStream_t stream) {
   kp.min_chunk = (a.min_chunk_tokens + 15) / 16;
   kp.tiles_per_block = a.pool.block_size / 16;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
+  kp.key_mask = a.key_mask;
+  kp.key_mask_stride_seq = a.key_mask_stride_seq;
+  kp.key_mask_stride_head = a.key_mask_stride_head;
+  if (a.key_mask != nullptr && a.dtype != IC_DTYPE_F32) return IC_ERR_UNSUPPORTED;
   switch (a.dtype) {
     case IC_DTYPE_BF16: return launch_hd<Bf16>(kp, a.hd, a.dtype, stream);
     case IC_DTYPE_F16: return launch_hd<F16>(kp, a.hd, a.dtype, stream);

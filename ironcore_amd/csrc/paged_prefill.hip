@@ -79,9 +79,21 @@ struct PrefillKP {
   int n_qtiles;     // query tiles per chunk (grid sizing)
   int causal;
   float scale_log2e;
+  // General attention mask (MASK variant): byte (sequence i, head h, chunk row r, key j) at
+  // mask[i*mask_stride_seq + h*mask_stride_head + r*mask_stride_row + j], nonzero = visible.
+  const uint8_t *mask;
+  int64_t mask_stride_seq;
+  int64_t mask_stride_head;
+  int64_t mask_stride_row;
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
+// Raw score of a key the mask hides.  The reference fills hidden scores with the FINITE minimum
+// of the element type (attention.py:66,115-117), not -inf: beside any visible key the hidden ones
+// get probability 0 either way, but a row with no visible key at all becomes a uniform average of
+// V over the whole context.  A power of two, so that its product with the scale is exact and the
+// exponent of a fully hidden row is exactly 0.
+constexpr float kHiddenScore = -0x1p100f;
 
 // x of this lane and x of lane ^ 32, as a pair (v_permlane32_swap: a vector-ALU
 // exchange, where a shuffle would be an LDS operation and share its counter).
@@ -131,7 +143,9 @@ constexpr int kBM = kPrefillWaves * 32;   // query rows per workgroup
 
 // SINGLE: every sequence is one pool block (a dense [b, sk, gn, hd] tensor
 // viewed as a pool); otherwise blocks are a power of two >= 16 tokens long.
-template <class M, int HD, bool SINGLE>
+// MASK: visibility comes from a byte mask instead of the causal rule; every
+// query row walks all L keys and a chunk may be longer than its context.
+template <class M, int HD, bool SINGLE, bool MASK>
 __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const PrefillKP p) {
   using T = typename M::T;
   constexpr int KS = HD / 16;          // k-steps of the QK contraction
@@ -192,10 +206,18 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   }
   const int h = kvh * p.group + r / p.n_qtiles;
   const int q0 = (p.n_qtiles - 1 - r % p.n_qtiles) * kBM;
+  const bool causal = !MASK && p.causal;
   if (L < 0) L = 0;
-  if (C > L) C = L;  // a chunk cannot be longer than its context
+  if (causal && C > L) C = L;  // under the causal rule a chunk cannot be longer than its context
   if (q0 >= C) return;
-  const int P = L - C;  // cached prefix
+  if (L == 0) {  // query rows without any key (not under the causal rule): zero rows
+    const int rows = C - q0 < kBM ? C - q0 : kBM;
+    for (int idx = threadIdx.x; idx < rows * (HD / 8); idx += kPrefillThreads)
+      store16(p.out + ((q_lo + q0 + idx / (HD / 8)) * p.out_stride_token + (int64_t)h * HD + (idx % (HD / 8)) * 8) * 2,
+              Vec16{{0u, 0u, 0u, 0u}});
+    return;
+  }
+  const int P = L - C;  // cached prefix (causal rule only)
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -206,7 +228,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // ---- query rows: registers for the whole sweep, as MFMA B operands ------------
   const int my_q = q0 + wave * 32 + n;
   const int qrow = my_q < C ? my_q : C - 1;
-  const int limit = p.causal ? P + qrow : L - 1;  // last key this query row may see
+  const int limit = causal ? P + qrow : L - 1;  // last key this query row may see
   Vec16 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
@@ -219,12 +241,12 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[ob][i] = 0.f;
 
-  int kv_end = p.causal ? P + q0 + kBM : L;  // keys any row of this workgroup can see
+  int kv_end = causal ? P + q0 + kBM : L;  // keys any row of this workgroup can see
   kv_end = kv_end < L ? kv_end : L;
   const int n_tiles = (kv_end + kBN - 1) / kBN;
   // tiles this wave's rows reach (the causal diagonal cuts the later ones off;
   // a wave whose rows all lie past the end of the chunk has nothing to compute)
-  int my_end = p.causal ? P + q0 + wave * 32 + 32 : L;
+  int my_end = causal ? P + q0 + wave * 32 + 32 : L;
   my_end = my_end < kv_end ? my_end : kv_end;
   const int my_tiles = (my_end > 0 && q0 + wave * 32 < C) ? (my_end + kBN - 1) / kBN : 0;
 
@@ -338,7 +360,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   auto softmax = [&](int tile) {
     // s[tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n)
     const int tok_base = tile * kBN + 4 * hh;
-    const bool need_mask = p.causal ? (tile * kBN + kBN - 1 > P + q0 + wave * 32) : (tile * kBN + kBN > L);
+    const bool need_mask = causal ? (tile * kBN + kBN - 1 > P + q0 + wave * 32) : (tile * kBN + kBN > L);
     if (need_mask) {  // tiles that touch the causal diagonal (or the context end)
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
@@ -346,6 +368,18 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
         for (int i = 0; i < 16; ++i) {
           const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
           s[tb][i] = tok > limit ? kNegInf : s[tb][i];
+        }
+    }
+    if constexpr (MASK) {  // keys the caller's mask hides from this lane's query row
+      const uint8_t *mrow = p.mask + (int64_t)seq * p.mask_stride_seq + (int64_t)h * p.mask_stride_head +
+                            (int64_t)qrow * p.mask_stride_row;
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
+          const bool hidden = tok <= limit && mrow[tok] == 0;
+          s[tb][i] = hidden ? kHiddenScore : s[tb][i];
         }
     }
     // Row maximum on the raw scores (the scale is positive), one exchange
@@ -521,7 +555,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   }
 }
 
-template <class M, bool SINGLE>
+template <class M, bool SINGLE, bool MASK>
 int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
   kp.n_qtiles = (a.max_chunk_len + kBM - 1) / kBM;
   const int64_t slices = (kp.n_units + kXcds - 1) / kXcds;
@@ -530,10 +564,10 @@ int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)wgs);
   switch (a.hd) {
     case 64:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 64, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 64, SINGLE, MASK>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     case 128:
-      hipLaunchKernelGGL((paged_prefill_kernel<M, 128, SINGLE>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 128, SINGLE, MASK>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
     default:
       return IC_ERR_UNSUPPORTED;
@@ -544,9 +578,11 @@ int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
 template <class M>
 int launch_mode(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
   // A one-column block table means one block per sequence, of any length.
-  if (a.block_table_stride == 1) return launch_hd<M, true>(kp, a, stream);
+  const bool masked = a.mask != nullptr;
+  if (a.block_table_stride == 1)
+    return masked ? launch_hd<M, true, true>(kp, a, stream) : launch_hd<M, true, false>(kp, a, stream);
   if (kp.block_shift < 4) return IC_ERR_UNSUPPORTED;  // power-of-two blocks of >= 16 tokens
-  return launch_hd<M, false>(kp, a, stream);
+  return masked ? launch_hd<M, false, true>(kp, a, stream) : launch_hd<M, false, false>(kp, a, stream);
 }
 
 }  // namespace
@@ -577,6 +613,10 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   kp.n_qtiles = 0;
   kp.causal = a.causal;
   kp.scale_log2e = a.scale * 1.4426950408889634f;
+  kp.mask = a.mask;
+  kp.mask_stride_seq = a.mask_stride_seq;
+  kp.mask_stride_head = a.mask_stride_head;
+  kp.mask_stride_row = a.mask_stride_row;
   if ((int64_t)a.max_chunk_len >= (int64_t)65535 * 128 || a.hn > 65535 || a.n_seqs > 65535)
     return IC_ERR_UNSUPPORTED;
   switch (a.dtype) {

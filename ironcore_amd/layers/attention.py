@@ -23,6 +23,7 @@ there is no torch fallback.
 """
 from __future__ import annotations
 
+import weakref
 from dataclasses import dataclass
 from typing import Optional
 
@@ -31,6 +32,10 @@ from torch import nn
 
 from .. import paged_ops
 from .module import BaseModule, get_model_dtype
+
+
+# attention_mask tensor -> what _classify_mask found for it: id -> (weak reference, (version, shapes), kind, bytes)
+_MASK_CLASSES: dict = {}
 
 
 @dataclass
@@ -96,25 +101,55 @@ class Attention(BaseModule):
         if self.training and self.config.model.dropout_attn > 0.0:
             raise NotImplementedError("attention dropout is a training feature; the paged "
                                       "kernels implement the inference path (dropout_attn == 0 or eval())")
+        if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+            # The reference's layer is differentiable (its tests backpropagate through it,
+            # tests/test_attention.py:391-426); the HIP kernels are forward only and their output
+            # carries no graph, so a backward pass would silently leave attention and the Q/K/V
+            # projections without gradient.
+            raise NotImplementedError(
+                "the HIP attention path is forward only: query/key/value require grad and autograd is "
+                "recording; call it under torch.no_grad() / torch.inference_mode() or on detached tensors")
 
-    def _mask_is_causal(self, attention_mask, sq, sk) -> bool:
-        """True for the lower-triangular mask the reference model builds
-        (ironcore/language_model.py:109-114,159), shifted when sq < sk; None
-        means every key is visible.  Anything else is rejected: the kernels
-        implement those two patterns."""
+    def _classify_mask(self, attention_mask, b, sq, sk, hn):
+        """What the kernels have to do for this mask (0 = hidden, broadcastable
+        to [b, hn, sq, sk], attention.py:115-117): ``("none", None)`` when every
+        key is visible, ``("causal", None)`` for the lower-triangular pattern the
+        reference model builds (ironcore/language_model.py:109-114,159; shifted
+        when sq < sk), else ``("general", bytes)`` with the mask as a uint8
+        ``[1 or b, 1 or hn, sq, sk]`` tensor for the masked kernels.
+
+        Telling the patterns apart needs a look at the values (one device
+        synchronisation); the answer is remembered per mask TENSOR (identity
+        and version counter), so a model that hands one mask to all its layers
+        pays once per forward pass, not once per layer."""
         if attention_mask is None:
-            return False
-        i = torch.arange(sq, device=attention_mask.device).unsqueeze(1)
-        j = torch.arange(sk, device=attention_mask.device).unsqueeze(0)
-        want = (j <= (sk - sq) + i)
-        got = attention_mask != 0
-        if got.shape[-2:] != (sq, sk):
-            raise ValueError(f"attention_mask must end in [{sq}, {sk}], got {tuple(attention_mask.shape)}")
-        if bool((got == want).all()):
-            return True
-        if bool(got.all()):
-            return False
-        raise NotImplementedError("only the causal mask (or no mask) is supported by the HIP attention path")
+            return "none", None
+        hit = _MASK_CLASSES.get(id(attention_mask))
+        if hit is not None and hit[0]() is attention_mask and hit[1] == (attention_mask._version, b, sq, sk, hn):
+            return hit[2], hit[3]
+        m = attention_mask
+        while m.dim() < 4:
+            m = m.unsqueeze(0)
+        if m.dim() != 4 or m.shape[-2:] != (sq, sk) or m.shape[0] not in (1, b) or m.shape[1] not in (1, hn):
+            raise ValueError(f"attention_mask must be broadcastable to [{b}, {hn}, {sq}, {sk}], "
+                             f"got {tuple(attention_mask.shape)}")
+        visible = m != 0
+        i = torch.arange(sq, device=m.device).unsqueeze(1)
+        j = torch.arange(sk, device=m.device).unsqueeze(0)
+        want = j <= (sk - sq) + i
+        flags = torch.stack([visible.all(), (visible == want).all()]).tolist()   # the one synchronisation
+        if flags[0]:
+            kind, data = "none", None
+        elif flags[1] and sq <= sk:
+            kind, data = "causal", None
+        else:
+            kind, data = "general", visible.to(torch.uint8).contiguous()
+        if len(_MASK_CLASSES) > 64:
+            for key in [k for k, v in _MASK_CLASSES.items() if v[0]() is None]:
+                del _MASK_CLASSES[key]
+        _MASK_CLASSES[id(attention_mask)] = (weakref.ref(attention_mask), (attention_mask._version, b, sq, sk, hn),
+                                             kind, data)
+        return kind, data
 
     # ------------------------------------------------------------------ forward
     def forward(self, query, key, value, attention_mask=None, *, kv_cache=None, attn_metadata=None,
@@ -135,9 +170,10 @@ class Attention(BaseModule):
     def _dense(self, query, key, value, attention_mask):
         b, sq, hn, hd = query.shape
         sk, gn = key.shape[1], key.shape[2]
-        causal = self._mask_is_causal(attention_mask, sq, sk)
+        kind, mask = self._classify_mask(attention_mask, b, sq, sk, hn)
+        causal = kind == "causal"
         if query.dtype == torch.float32:
-            return self._dense_fp32(query, key, value, causal)
+            return self._dense_fp32(query, key, value, causal, mask)
         key, value = key.contiguous(), value.contiguous()
         # one pool block per sequence: [b, gn, sk, hd] view of the [b, sk, gn, hd] rows
         k_pool, v_pool = key.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)
@@ -146,7 +182,7 @@ class Attention(BaseModule):
         ctx = torch.full((b,), sk, dtype=torch.int32, device=dev)
         cu = torch.arange(0, (b + 1) * sq, sq, dtype=torch.int32, device=dev)
         out = paged_ops.paged_prefill(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx, cu, sq,
-                                      causal=causal, scale=1.0 / self.scale_factor)
+                                      causal=causal, scale=1.0 / self.scale_factor, mask=mask)
         return out.view(b, sq, hn * hd)
 
     def _ragged_chunks(self, query, k_pool, v_pool, meta, rows, scale):
@@ -164,9 +200,12 @@ class Attention(BaseModule):
         out.index_copy_(0, rows, got)
         return out.view(b, sq, hn * hd)
 
-    def _dense_fp32(self, query, key, value, causal):
+    def _dense_fp32(self, query, key, value, causal, mask=None):
         """fp32 has no MFMA path: every query row runs as one decode-kernel
-        sequence over the keys it may see (fp32 loads, fp32 arithmetic)."""
+        sequence over the keys it may see (fp32 loads, fp32 arithmetic); a
+        general mask travels as one key-mask row per query row.  K and V are
+        streamed once per query ROW, so this costs sq times the traffic of the
+        16-bit kernel: it is there for exactness at small sizes, not speed."""
         b, sq, hn, hd = query.shape
         sk, gn = key.shape[1], key.shape[2]
         dev = query.device
@@ -181,7 +220,7 @@ class Attention(BaseModule):
         return _fp32_rows_via_decode(query, k_pool, v_pool,
                                      torch.arange(b, dtype=torch.int32, device=dev).unsqueeze(1),
                                      torch.full((b,), sk, dtype=torch.int32, device=dev), sk, causal,
-                                     1.0 / self.scale_factor)
+                                     1.0 / self.scale_factor, mask)
 
     def _paged(self, query, key, value, kv_cache, meta, rotary_pos_emb=None):
         if meta is None:
@@ -236,14 +275,23 @@ def _ragged_rows_fp32(query_rows, k_pool, v_pool, meta, scale):
     return paged_ops.paged_decode(query_rows, k_pool, v_pool, tables, ctx, meta.max_context_len, scale=scale)
 
 
-def _fp32_rows_via_decode(query, k_pool, v_pool, block_tables, context_lens, max_context_len, causal, scale):
+def _fp32_rows_via_decode(query, k_pool, v_pool, block_tables, context_lens, max_context_len, causal, scale,
+                          mask=None):
     """Chunk attention in fp32: query row r of sequence i becomes one
     decode-kernel sequence with context_lens[i] - (sq - 1 - r) visible tokens
-    (all of them when not causal), sharing sequence i's block-table row."""
+    (all of them when not causal), sharing sequence i's block-table row.
+    ``mask`` (uint8 [1 or b, 1 or hn, sq, sk]) hides keys per query row."""
     b, sq, hn, hd = query.shape
     dev = query.device
     rows = torch.arange(b, device=dev).repeat_interleave(sq)
     tables = block_tables.index_select(0, rows)
+    if mask is not None:
+        mh, sk = mask.shape[1], mask.shape[3]
+        key_mask = mask.expand(b, mh, sq, sk).permute(0, 2, 1, 3).reshape(b * sq, mh, sk).contiguous()
+        ctx = context_lens.index_select(0, rows).contiguous()
+        out = paged_ops.paged_decode(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx,
+                                     max_context_len, scale=scale, key_mask=key_mask)
+        return out.view(b, sq, hn * hd)
     if causal:
         back = (sq - 1 - torch.arange(sq, device=dev, dtype=torch.int32)).repeat(b)
         ctx = (context_lens.index_select(0, rows) - back).to(torch.int32)

@@ -146,8 +146,14 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
                  block_tables: torch.Tensor, context_lens: torch.Tensor, max_context_len: int,
                  scale: float | None = None, out: torch.Tensor | None = None,
                  min_chunk_tokens: int = 0, cohort_size: int = 1,
-                 cohort_shared_blocks: torch.Tensor | None = None) -> torch.Tensor:
+                 cohort_shared_blocks: torch.Tensor | None = None,
+                 key_mask: torch.Tensor | None = None) -> torch.Tensor:
     """One query token per sequence.  ``query`` ``[b, hn, hd]`` -> ``[b, hn*hd]``.
+
+    ``key_mask`` (fp32 only; uint8 ``[b, 1 or hn, >= max_context_len]``,
+    contiguous): 0 hides a key from that sequence's query (head); hidden keys
+    get the reference's finite fill value, so a query that sees nothing
+    averages V over its context.
 
     ``max_context_len`` is a host-side upper bound on ``context_lens`` (no
     device synchronisation is needed to launch).  ``min_chunk_tokens`` is the
@@ -199,6 +205,24 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     if need == 0 and b > 0:
         raise ValueError(f"cohort_size {cohort_size} with {hn // gn} query heads per KV head is not supported")
     ws = _workspace.get(dev, need)
+    if key_mask is not None:
+        if key_mask.dtype != torch.uint8 or key_mask.dim() != 3 or key_mask.shape[0] != b \
+                or key_mask.shape[1] not in (1, hn) or key_mask.shape[2] < max_context_len \
+                or not key_mask.is_contiguous() or key_mask.device != dev:
+            raise ValueError(f"key_mask must be a contiguous uint8 [{b}, 1 or {hn}, >= {max_context_len}] tensor")
+        if cohort_size != 1:
+            raise ValueError("key_mask and cohorts do not combine")
+        with torch.cuda.device(dev):
+            rc = lib.ic_paged_decode_masked(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                            k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                            block_tables.data_ptr(), block_tables.stride(0),
+                                            context_lens.data_ptr(), b, hn, gn, hd, bs, nb, max_context_len,
+                                            float(scale), min_chunk_tokens, key_mask.data_ptr(),
+                                            key_mask.stride(0), key_mask.stride(1) if key_mask.shape[1] > 1 else 0,
+                                            ws.data_ptr(), ws.numel(),
+                                            _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+        _lib.check("ic_paged_decode_masked", rc)
+        return out
     with torch.cuda.device(dev):
         rc = lib.ic_paged_decode_shared(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
                                         k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
@@ -278,11 +302,17 @@ def shared_prefix_blocks(block_tables, context_lens, block_size: int, cohort_siz
 def paged_prefill(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                   block_tables: torch.Tensor, context_lens: torch.Tensor,
                   cu_seqlens_q: torch.Tensor, max_chunk_len: int, causal: bool = True,
-                  scale: float | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+                  scale: float | None = None, out: torch.Tensor | None = None,
+                  mask: torch.Tensor | None = None) -> torch.Tensor:
     """Chunked prefill.  ``query`` is the flat ``[n_tokens, hn, hd]``
     concatenation of the sequences' new chunks (chunk ``i`` = rows
     ``cu_seqlens_q[i]:cu_seqlens_q[i+1]``); the chunk's K/V are already in the
-    pool and ``context_lens[i]`` counts prefix + chunk.  -> ``[n_tokens, hn*hd]``."""
+    pool and ``context_lens[i]`` counts prefix + chunk.  -> ``[n_tokens, hn*hd]``.
+
+    ``mask`` (uint8 ``[1 or n_seqs, 1 or hn, >= max_chunk_len, >= max context]``,
+    last dimension contiguous) replaces the causal rule: byte (i, h, r, j) == 0
+    hides key j from row r of chunk i (head h).  Hidden keys get the
+    reference's finite fill value: a row that sees nothing averages V."""
     lib = _lib.load()
     dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens, cu_seqlens_q)
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
@@ -310,6 +340,24 @@ def paged_prefill(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
         raise ValueError("out must be [n_tokens, hn*hd] in the query dtype with contiguous rows")
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
+    if mask is not None:
+        if mask.dtype != torch.uint8 or mask.dim() != 4 or mask.shape[0] not in (1, n_seqs) \
+                or mask.shape[1] not in (1, hn) or mask.shape[2] < max_chunk_len or mask.stride(3) != 1 \
+                or mask.device != dev:
+            raise ValueError(f"mask must be uint8 [1 or {n_seqs}, 1 or {hn}, >= {max_chunk_len}, keys] on {dev} "
+                             "with a contiguous last dimension")
+        with torch.cuda.device(dev):
+            rc = lib.ic_paged_prefill_masked(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
+                                             k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,
+                                             block_tables.data_ptr(), block_tables.stride(0),
+                                             context_lens.data_ptr(), cu_seqlens_q.data_ptr(), n_seqs,
+                                             int(max_chunk_len), hn, gn, hd, bs, nb, float(scale),
+                                             mask.data_ptr(),
+                                             mask.stride(0) if mask.shape[0] > 1 else 0,
+                                             mask.stride(1) if mask.shape[1] > 1 else 0, mask.stride(2),
+                                             _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+        _lib.check("ic_paged_prefill_masked", rc)
+        return out
     with torch.cuda.device(dev):
         rc = lib.ic_paged_prefill(out.data_ptr(), out.stride(0), query.data_ptr(), query.stride(0),
                                   k_pool.data_ptr(), v_pool.data_ptr(), sb, sh, st,

@@ -18,3 +18,16 @@ def gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How often the randomized tests leaned on the short-context allowance of parity_bars.py."""
+    try:
+        from parity_bars import RELAX_BELOW_CTX, TALLY
+    except ImportError:
+        return
+    if TALLY["cases"]:
+        terminalreporter.write_line(
+            f"parity_bars: {TALLY['cases']} randomized cases; {TALLY['relaxed_elements']} elements in "
+            f"{TALLY['relaxed_cases']} cases passed the stated bar only by the oracle's own distance to float64 "
+            f"(allowed below {RELAX_BELOW_CTX} visible tokens only)")

@@ -55,7 +55,7 @@ def test_random_layer_and_cache_traffic(gpu, seed, hn, gn, hd, block):
             causal = (torch.arange(t).unsqueeze(0) <= (t - c) + torch.arange(c).unsqueeze(1)).view(1, 1, c, t)
             ref = dense_attention(q[i:i + 1, :c], K.unsqueeze(0), V.unsqueeze(0), causal)
             truth = dense_attention(q[i:i + 1, :c].double(), K.unsqueeze(0).double(), V.unsqueeze(0).double(), causal)
-            hold(out[i:i + 1, :c], ref, truth, torch.bfloat16, f"sequence {sid} ({t} tokens, {c} new)")
+            hold(out[i:i + 1, :c], ref, truth, torch.bfloat16, t - c + 1, f"sequence {sid} ({t} tokens, {c} new)")
 
     calls = 0
     for it in range(60):

@@ -232,3 +232,27 @@ def test_prepare_with_chunks_of_unequal_length():
     assert meta.positions.view(3, 5)[0].tolist() == [10, 11, 12, 0, 0]
     with pytest.raises(ValueError):
         cache.prepare([a, b], [1, 2], cohort_size=2)
+
+
+def test_attention_refuses_inputs_that_require_grad():
+    """The reference's layer is differentiable (tests/test_attention.py:391-426
+    backpropagates through it); the HIP path is forward only and says so
+    instead of returning a tensor without a graph.  Raised on the host, before
+    anything touches a device."""
+    import pytest
+    import torch
+    from ironcore_amd import config as ic_config
+    from ironcore_amd.layers import Attention
+    cfg = ic_config.MainConfig(model=ic_config.ModelConfig(d_model=128, num_attention_heads=2,
+                                                           num_attention_groups=2, head_dim=64, dropout_attn=0.0,
+                                                           precision="bf16"),
+                               trainer=ic_config.TrainerConfig(use_flash_attn=False))
+    attn = Attention(cfg)
+    q = torch.randn(1, 4, 2, 64, requires_grad=True)
+    k, v = torch.randn(1, 4, 2, 64), torch.randn(1, 4, 2, 64)
+    for args in ((q, k, v), (k, q, v), (k, v, q)):
+        with pytest.raises(NotImplementedError, match="forward only"):
+            attn(*args)
+    with torch.no_grad():                            # not recording: passes the check (and then needs a GPU)
+        with pytest.raises(RuntimeError, match="GPU only"):
+            attn(q, k, v)
