@@ -17,14 +17,17 @@
 //    operands.  Workgroup ids are laid out so that all tiles and heads that
 //    read the same K/V rows run on one XCD and share its L2.
 //  * K/V are walked in tiles of 64 tokens (4 pool blocks).  Four waves stage
-//    K and four stage V, each one 16-row group of every tile: its 16-byte
-//    pieces are fetched through the block table TWO tiles ahead (one table
-//    entry per wave and tile, a scalar load issued before the step's
-//    softmax), then parked in double-buffered LDS, row-major ([token][dim],
-//    padded pitch).  Every load is unconditional (addresses are clamped into
-//    the sequence's blocks, rows past the context are zeroed when parked), so
-//    the waits on the memory counter are exact and a tile's latency hides
-//    behind two tiles of arithmetic.
+//    K and four stage V, each one 16-row group of every tile, fetched through
+//    the block table (one table entry per wave and tile, a scalar load issued
+//    before the step's softmax) STRAIGHT INTO LDS (global_load_lds: the data
+//    never passes through registers, and no LDS write instruction competes
+//    with the operand reads), two to three tiles ahead, into four LDS buffers
+//    per pool, row-major ([token][dim]), unpadded, 16-byte chunks swizzled
+//    within a row so that the operand reads stay free of bank conflicts.
+//    Every load is unconditional (addresses are clamped into the sequence's
+//    blocks; rows of a V tile past the context are overwritten with zeros
+//    once they have landed), so the waits on the memory counter are exact and
+//    a tile's latency hides behind two tiles of arithmetic.
 //  * Two-sided schedule: the waves of a SIMD run half a tile apart, one in
 //    its matrix step while the other is in its vector (softmax) step, with a
 //    workgroup barrier between steps; see the loop at the end of the kernel.
@@ -140,6 +143,7 @@ constexpr int kPrefillThreads = kPrefillWaves * kWave;
 constexpr int kXcds = 8;
 constexpr int kBN = 64;                   // tokens per K/V tile
 constexpr int kBM = kPrefillWaves * 32;   // query rows per workgroup
+constexpr int kStageBuffers = 4;          // LDS buffers per pool: a tile is fetched three tiles ahead
 
 // SINGLE: every sequence is one pool block (a dense [b, sk, gn, hd] tensor
 // viewed as a pool); otherwise blocks are a power of two >= 16 tokens long.
@@ -154,12 +158,21 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   constexpr int CPR = HD / 8;          // 16-byte chunks per token row
   constexpr int WR = kWave / CPR;      // token rows one load instruction of a wave covers
   constexpr int NST = 16 / WR;         // loads (16-byte pieces) per lane and staged tile
-  constexpr int KP = HD * 2 + 16;      // K tile pitch in bytes (bank-conflict-free b128 reads)
-  constexpr int VP = HD * 2 + 64;      // V tile pitch in bytes (conflict-free transposing reads)
-  static_assert(kBN == 64 && 16 % WR == 0, "tile staging shape");
+  constexpr int ROWB = HD * 2;         // bytes of one token row; LDS tiles are unpadded [token][dim]
+  constexpr int NB = kStageBuffers;    // LDS buffers per pool
+  static_assert(kBN == 64 && 16 % WR == 0 && (CPR == 8 || CPR == 16), "tile staging shape");
 
-  __shared__ __attribute__((aligned(16))) char s_k[2][kBN * KP];
-  __shared__ __attribute__((aligned(16))) char s_v[2][kBN * VP];
+  // A tile reaches LDS straight from memory (global_load_lds: no registers, no LDS write
+  // instruction), 1 KiB per wave and load, lane l's 16 bytes at byte 16*l of that KiB.  Rows are
+  // therefore unpadded, and what keeps the operand reads free of bank conflicts is a swizzle:
+  // 16-byte chunk c of tile row r lives in slot c ^ swz(r) of its row (the lane that fills a slot
+  // simply fetches the chunk that belongs there).  K (read as whole 16-byte chunks, 16 rows per
+  // access): swz = r % 16 (head dim 128), (r / 2) % 8 (head dim 64).  V (read by the transposing
+  // 8-byte reads, 4 rows x 64 bytes per access): swz = 4 * (r % 4), resp. 4 * ((r / 2) % 2).
+  __shared__ __attribute__((aligned(1024))) char s_k[NB][kBN * ROWB];
+  __shared__ __attribute__((aligned(1024))) char s_v[NB][kBN * ROWB];
+  auto swz_k = [](int r) { return CPR == 16 ? (r & 15) : ((r >> 1) & 7); };
+  auto swz_v = [](int r) { return CPR == 16 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2); };
 
   // XCD-aware placement.  Workgroups are dealt to the 8 XCDs round-robin by
   // their linear id, and each XCD has its own L2.  All workgroups that read
@@ -250,30 +263,39 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   my_end = my_end < kv_end ? my_end : kv_end;
   const int my_tiles = (my_end > 0 && q0 + wave * 32 < C) ? (my_end + kBN - 1) / kBN : 0;
 
-  // ---- tile staging: global -> registers -> LDS -----------------------------------
+  // ---- tile staging: memory -> LDS ---------------------------------------------------
   // A wave stages one 16-row group of every tile (group wave & 3) of ONE pool:
   // the waves of side 0 stage K, those of side 1 stage V.  Pool blocks are a
   // power of two >= 16 rows long (or the sequence is a single block), so a
   // group lies inside one block: one table entry and one base address per wave
-  // and tile, scalar work, and a lane only adds fixed offsets.  (A wave issues
-  // an instruction every four to five cycles whatever its kind, so the
-  // address arithmetic of the staging is paid in the same currency as the
-  // softmax beside it: with two passes over both pools per thread it cost as
-  // much as the softmax.)  Nothing here is conditional: a tile index past the
-  // sweep is clamped to the last tile, a block index past the sequence to its
-  // last block (whose 16-row groups are allocated whether filled or not), and
-  // in SINGLE mode a row past the context to the last row.
+  // and tile, scalar work, and a lane only adds fixed offsets.  Nothing here is
+  // conditional: a tile index past the sweep is clamped to the last tile, a
+  // block index past the sequence to its last block (whose 16-row groups are
+  // allocated whether filled or not), and in SINGLE mode a row past the context
+  // to the last row; so every wave has the same number of loads in flight at the
+  // same point of the program and the waits on the memory counter are exact.
+  // The loads are written as inline assembly: to the compiler an LDS-writing
+  // load is something every later LDS read must wait for, which would serialise
+  // the prefetch; here the order is kept by hand (landed() before the workgroup
+  // barrier that precedes a tile's first read).
   const int grp = wave & 3;
-  const int cc = lane % CPR;
-  const int rsub = lane / CPR;
+  const int cc = lane % CPR;    // LDS slot (16-byte chunk of the row) this lane fills
+  const int rsub = lane / CPR;  // row within the rows one load covers
   const char *stage_pool = side == 0 ? p.k_pool : p.v_pool;
-  const int stage_pitch = side == 0 ? KP : VP;
-  const uint32_t thr_off = (uint32_t)((rsub * p.stride_token + cc * 8) * 2);
-  const int64_t step_off = (int64_t)WR * p.stride_token * 2;
   const int64_t head_off = (int64_t)kvh * p.stride_head;
   const int last_blk = SINGLE ? 0 : (L - 1) >> p.block_shift;
   typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
   const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
+  // byte offset, from the group's first row, of the chunk lane l fetches with load i: row
+  // i*WR + rsub of the group, and the chunk whose place in that row is this lane's slot
+  uint32_t lane_src[NST];
+#pragma unroll
+  for (int i = 0; i < NST; ++i) {
+    const int r = i * WR + rsub;  // (a group starts at a multiple of 16 rows: r stands for the tile row)
+    const int chunk = cc ^ (side == 0 ? swz_k(r) : swz_v(r));
+    lane_src[i] = (uint32_t)((int64_t)r * p.stride_token * 2 + chunk * 16);
+  }
+  const uint32_t lds_pool = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)(side == 0 ? &s_k[0][0] : &s_v[0][0]);
   auto clamp_tile = [&](int tile) { return tile < n_tiles ? tile : n_tiles - 1; };
   auto lookup = [&](int tile, int32_t &ent) {
     const int first = clamp_tile(tile) * kBN + 16 * grp;  // this wave's first row of the tile
@@ -281,56 +303,67 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     blk = blk < last_blk ? blk : last_blk;
     ent = table_row[blk];
   };
-  auto fetch_rows = [&](int tile, int32_t ent, Vec16 *st) {
+  // Issue the loads of this wave's group of `tile` into the tile's LDS buffer.
+  auto fetch_rows = [&](int tile, int32_t ent) {
     const int first = clamp_tile(tile) * kBN + 16 * grp;
     int64_t phys = ent;
     // A corrupt table entry must not become an out-of-pool address.
     phys = phys < 0 ? 0 : phys;
     phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
+    const uint32_t dst = lds_pool + (uint32_t)((tile & (NB - 1)) * (kBN * ROWB) + 16 * grp * ROWB);
     if (SINGLE) {
+      const char *base = stage_pool + (phys * p.stride_block + head_off) * 2;
 #pragma unroll
       for (int i = 0; i < NST; ++i) {
         int row = first + rsub + i * WR;
         row = row < L ? row : L - 1;
-        st[i] = load16(stage_pool + (phys * p.stride_block + head_off + (int64_t)row * p.stride_token + cc * 8) * 2);
+        const int chunk = cc ^ (side == 0 ? swz_k(i * WR + rsub) : swz_v(i * WR + rsub));
+        const char *src = base + (int64_t)row * p.stride_token * 2 + chunk * 16;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(dst + i * WR * ROWB), "v"(src) : "memory", "m0");
       }
     } else {
       const int rem = first & (p.block_size - 1);
-      const char *base = stage_pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2 + thr_off;
+      const char *base = stage_pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2;
 #pragma unroll
-      for (int i = 0; i < NST; ++i) st[i] = load16(base + i * step_off);
+      for (int i = 0; i < NST; ++i)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(dst + i * WR * ROWB), "v"(lane_src[i]), "s"(base) : "memory", "m0");
     }
   };
-  const int park_at = (16 * grp + rsub) * stage_pitch + cc * 16;
-  auto park_rows = [&](int tile, const Vec16 *st) {
-    if (tile >= n_tiles) return;
-    char *buf = (side == 0 ? s_k[tile & 1] : s_v[tile & 1]) + park_at;
-    const int row = tile * kBN + 16 * grp + rsub;
-    if (tile * kBN + 16 * grp + 16 <= L) {  // the whole group lies inside the context (wave-uniform)
+  // The loads of `tile` have arrived (everything but the `younger` loads issued after them); rows
+  // of a V tile past the context become zeros (their probabilities are zeros, but 0 x NaN is not:
+  // unused pool slots may hold anything).  The workgroup barrier that follows makes the tile
+  // readable.
+  auto landed = [&](int tile, int younger_tiles) {
+    if (younger_tiles == 0)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (younger_tiles == 1)
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NST) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NST) : "memory");
+    if (side == 1 && tile < n_tiles && tile * kBN + 16 * grp + 16 > L) {
+      char *buf = s_v[tile & (NB - 1)] + 16 * grp * ROWB + lane * 16;
+      const int row = tile * kBN + 16 * grp + rsub;
 #pragma unroll
-      for (int i = 0; i < NST; ++i) store16(buf + i * WR * stage_pitch, st[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < NST; ++i) {
-        const bool live = row + i * WR < L;  // rows past the context are parked as zeros
-        Vec16 v;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) v.w[w] = live ? st[i].w[w] : 0u;
-        store16(buf + i * WR * stage_pitch, v);
-      }
+      for (int i = 0; i < NST; ++i)
+        if (row + i * WR >= L) store16(buf + i * WR * ROWB, Vec16{{0u, 0u, 0u, 0u}});
     }
   };
 
-  // per-lane LDS offsets
-  const int k_lane = n * KP + hh * 16;  // + tb*32*KP + ks*32
-  const int v_lane = (4 * hh + (lane & 15) / 4) * VP + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // per-lane LDS offsets of the operand reads (the swizzles above, seen from the reading side)
+  // K: row tb*32 + n, chunk 2*ks + hh  ->  (n*ROWB + 16*(hh ^ swz)) ^ 32*ks, + tb*32*ROWB
+  const int k_lane = n * ROWB + ((hh ^ swz_k(n)) << 4);
+  // V: rows kk*16 (+8) + 4*hh + q, bytes ob*64 + 32*bit4 + 8*(lane & 3)  ->  base ^ 64*ob
+  const int vq = (lane & 15) >> 2;
+  const int v_lane = (4 * hh + vq) * ROWB + ((swz_v(vq) >> 2) << 6) + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
 
   f32x16_t s[TB];        // S^T of the tile in flight: (token, query n)
   Vec16 pb[kBN / 16];    // its probabilities as MFMA B operands
 
   // ---- S^T = K Q^T ----------------------------------------------------------------
   auto scores = [&](int tile) {
-    const char *sk = s_k[tile & 1];
+    const char *sk = s_k[tile & (NB - 1)];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -339,7 +372,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     for (int tb = 0; tb < TB; ++tb) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const Vec16 a = load16(sk + k_lane + tb * 32 * KP + ks * 32);
+        const Vec16 a = load16(sk + (k_lane ^ (ks * 32)) + tb * 32 * ROWB);
         s[tb] = M::mma(a, qf[ks], s[tb]);
       }
     }
@@ -422,16 +455,16 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   };
   // ---- O^T += V^T P^T ---------------------------------------------------------------
   auto weighted_values = [&](int tile) {
-    const char *sv = s_v[tile & 1];
+    const char *sv = s_v[tile & (NB - 1)];
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob) {
 #pragma unroll
       for (int kk = 0; kk < kBN / 16; ++kk) {
-        const char *at = sv + v_lane + kk * 16 * VP + ob * 64;
+        const char *at = sv + (v_lane ^ (ob * 64)) + kk * 16 * ROWB;
         const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) s16x4_t *)(at));
         const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4_t *)(at + 8 * VP));
+            (__attribute__((address_space(3))) s16x4_t *)(at + 8 * ROWB));
         const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         o[ob] = M::mma(__builtin_bit_cast(Vec16, both), pb[kk], o[ob]);
       }
@@ -447,14 +480,13 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // busy at the same time.  A workgroup barrier ends each phase.
   //   side 0:  M(0) V(0) M(1) V(1) ... M(n) V(n)  -
   //   side 1:   -   M(0) V(0) M(1) ... V(n-1) M(n) V(n)
-  // LDS double buffers: K(k) and V(k-1) are read in phases 2k and 2k+1, so
-  // K(k+1) and V(k) are parked during those same two phases into the buffers
-  // K(k-1) and V(k-2) left: side 1 parks V(k) at the end of its vector step of
-  // phase 2k, side 0 parks K(k+1) at the end of its vector step of phase 2k+1.
-  // Registers: a thread carries two staged tiles of its pool; once a tile is
-  // parked its set is refilled with the tile two further on.
-  Vec16 stg[2][NST];
-  int32_t ent;  // table entry of the tile the next refill fetches
+  // LDS: four buffers per pool.  K(k) is read in phases 2k and 2k+1, V(k) in phases 2k+2 and
+  // 2k+3.  In its vector step k a wave first makes sure its group of tile k+1 has arrived (the
+  // barrier that ends the step publishes it: K(k+1) is first read in phase 2k+2, V(k+1) in phase
+  // 2k+4), then issues the loads of tile k+3 into the buffer tile k-1 left (last read in phase
+  // 2k-1 for K, 2k+1 for V: one barrier before the issue at the latest).  So a tile's loads are
+  // in flight for four phases, and a wave always has two tiles of its pool on the way.
+  int32_t ent;  // table entry of the tile the next vector step fetches
   auto matrix_step = [&](int k) {
     if (k >= 1 && k <= my_tiles) weighted_values(k - 1);
     if (k < my_tiles) {
@@ -466,15 +498,13 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
         for (int i = 0; i < 16; ++i) s[tb][i] = 0.f;
     }
   };
-  // Park staged tile `tile` from `set`, refill the set with tile + 2, then the
-  // softmax of tile j.  The memory operations go first (the staged data arrived
-  // two steps ago, the table entry of the refill was looked up in the previous
-  // step) and complete behind the softmax, which has no LDS or scalar-memory
-  // operation whose wait would include them.
-  auto vector_step = [&](int j, int tile, Vec16 *set) {
-    park_rows(tile, set);
-    fetch_rows(tile + 2, ent, set);
-    lookup(tile + 3, ent);  // for the next vector step, which refills with tile + 3
+  // Tile `tile` has arrived; fetch tile + 2; then the softmax of tile j.  The memory operations
+  // go first and complete behind the softmax, which has no LDS or scalar-memory operation whose
+  // wait would include them.
+  auto vector_step = [&](int j, int tile) {
+    landed(tile, 1);
+    fetch_rows(tile + 2, ent);
+    lookup(tile + 3, ent);  // for the next vector step, which fetches tile + 3
     if (j >= 0 && j < my_tiles) {
       softmax(j);
     } else {
@@ -482,57 +512,49 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
       for (int kk = 0; kk < kBN / 16; ++kk) pb[kk] = Vec16{{0u, 0u, 0u, 0u}};
     }
   };
-  // prologue: K(0) straight into LDS; side 0 then holds K(1), K(2), side 1 V(0), V(1)
+  // prologue: side 0 issues K(0), K(1), K(2) and waits for K(0); side 1 issues V(0), V(1)
   // (all table entries first, then all tiles: one round trip each, not one per tile)
   if (side == 0) {
     int32_t e0, e1, e2;
-    Vec16 first[NST];
     lookup(0, e0);
     lookup(1, e1);
     lookup(2, e2);
-    lookup(3, ent);  // the first vector step parks K(1) and refills with K(3)
-    fetch_rows(0, e0, first);
-    fetch_rows(1, e1, stg[0]);
-    fetch_rows(2, e2, stg[1]);
-    park_rows(0, first);
+    lookup(3, ent);  // the first vector step waits for K(1) and fetches K(3)
+    fetch_rows(0, e0);
+    fetch_rows(1, e1);
+    fetch_rows(2, e2);
+    landed(0, 2);
   } else {
     int32_t e0, e1;
     lookup(0, e0);
     lookup(1, e1);
-    lookup(2, ent);  // the first vector step parks V(0) and refills with V(2)
-    fetch_rows(0, e0, stg[0]);
-    fetch_rows(1, e1, stg[1]);
+    lookup(2, ent);  // the first vector step waits for V(0) and fetches V(2)
+    fetch_rows(0, e0);
+    fetch_rows(1, e1);
   }
   __syncthreads();
-  // Both sides pass the same number of barriers.  The loops are unrolled by two
-  // so that the register set of a staged tile is a compile-time choice.
+  // Both sides pass the same number of barriers.
   const int n_steps = (n_tiles + 2) & ~1;  // steps k = 0 .. n_steps-1 cover M(0..n_tiles), rounded up to even
   if (side == 0) {
-    for (int k = 0; k < n_steps; k += 2) {
+    for (int k = 0; k < n_steps; ++k) {
       matrix_step(k);
       __syncthreads();
-      vector_step(k, k + 1, stg[0]);  // parks K(k+1)
-      __syncthreads();
-      matrix_step(k + 1);
-      __syncthreads();
-      vector_step(k + 1, k + 2, stg[1]);
+      vector_step(k, k + 1);  // publishes K(k+1)
       __syncthreads();
     }
     __syncthreads();
   } else {
-    vector_step(-1, 0, stg[0]);  // parks V(0)
+    vector_step(-1, 0);  // publishes V(0)
     __syncthreads();
-    for (int k = 0; k < n_steps; k += 2) {
+    for (int k = 0; k < n_steps; ++k) {
       matrix_step(k);
       __syncthreads();
-      vector_step(k, k + 1, stg[1]);  // parks V(k+1)
-      __syncthreads();
-      matrix_step(k + 1);
-      __syncthreads();
-      vector_step(k + 1, k + 2, stg[0]);
+      vector_step(k, k + 1);  // publishes V(k+1)
       __syncthreads();
     }
   }
+  // every load this wave issued must have landed before its LDS is given up
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- normalise and store -------------------------------------------------------
   float l_a, l_b;
