@@ -48,6 +48,7 @@ namespace decode {
 namespace {
 
 constexpr float kLazyMaxSlack = 5.0f;  // log2 units
+constexpr int kLongRowTokens = 1024;     // longest context from which one workgroup per CU is launched
 
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
@@ -521,6 +522,17 @@ bool launch_variant(DecodeKP &kp, size_t lds_bytes, hipStream_t stream) {
     seen_bytes = lds_bytes;
   }
   int wgs = per_cu * device_cu_count();
+  // Long rows: one workgroup per CU.  A wave keeps two tiles (16 KiB at head dim 128) in flight,
+  // so one 4-wave workgroup per CU already has the bytes in flight that cover HBM's latency at its
+  // full rate; a second one adds queueing in the memory system and split-K segments (partials to
+  // write and merge, G times larger with G query heads per KV head) and no bandwidth: measured
+  // 2-3 % slower for G >= 2 at contexts of 1K-8K tokens (G = 1, whose partials are small, runs
+  // the same either way and keeps both workgroups).  With short rows the
+  // second workgroup pays: it hides the stalls of the row switches (query load, result write),
+  // 7 % on 256 sequences of 64-512 tokens.  Cohorts keep both: their two phases overlap across
+  // the workgroups of a CU.
+  if (!COOP && kp.cohort_size == 1 && kp.group >= 2 && kp.max_ctx >= kLongRowTokens && wgs > device_cu_count())
+    wgs = device_cu_count();
   if (wgs * NW > kp.max_waves) wgs = kp.max_waves / NW;
   kp.n_waves = wgs * NW;
   hipLaunchKernelGGL(kernel, dim3(wgs), dim3(NW * kWave), lds_bytes, stream, kp);
