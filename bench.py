@@ -73,6 +73,69 @@ def measured_traffic(workload, seed):
     return int(ent["hbm_bytes_per_launch"]), False
 
 
+DOMINANT_KERNEL = {"llama7b": "paged_decode_mfma_kernel", "llama70b": "paged_decode_mfma_kernel",
+                   "grpo": "paged_decode_mfma_kernel", "prefill": "paged_prefill_kernel"}
+COPY_BYTES = 1 << 30
+
+
+def traffic_record(prof_dir, seed):
+    """profiles/traffic.json from counter runs of this file (one counter per
+    run, --copy-calibration on): per workload, the dominant kernel's
+    FETCH_SIZE and WRITE_SIZE per dispatch (KiB, mean over its dispatches),
+    each scaled by what the same counter read for the 1 GiB device copy
+    (which reads and writes 1 GiB), as HBM bytes per launch."""
+    import csv
+    import glob
+    from ironcore_amd import build as ic_build
+
+    def per_dispatch(run_dir, counter, kernel):
+        files = glob.glob(os.path.join(run_dir, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            return None, None
+        mine, copies = [], []
+        for row in csv.DictReader(open(files[0])):
+            if row["Counter_Name"] != counter:
+                continue
+            name, val = row["Kernel_Name"], float(row["Counter_Value"])
+            if kernel in name:
+                mine.append(val)
+            elif "copy" in name.lower():
+                copies.append(val)
+        if not mine or not copies:
+            return None, None
+        # the calibration copies move 2^20 KiB each way; the counter reads that, or half of it (it
+        # counts in larger units on some paths), to within a percent
+        kib = COPY_BYTES / 1024.0
+        cal = [v for v in copies if abs(v / kib - 1) < 0.01 or abs(2 * v / kib - 1) < 0.01]
+        if not cal:
+            return None, None
+        return sum(mine) / len(mine), sum(cal) / len(cal)
+
+    rec = {"csrc_sha256": ic_build.csrc_digest(), "unit": "KiB per dispatch", "copy_bytes": COPY_BYTES,
+           "workloads": {}}
+    for workload, kernel in DOMINANT_KERNEL.items():
+        ent = {"kernel": kernel, "seed": seed}
+        total = 0.0
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            k, c = per_dispatch(os.path.join(prof_dir, f"pmc_{counter}_{workload}"), counter, kernel)
+            if k is None:
+                ent = None
+                break
+            scale = (COPY_BYTES / 1024.0) / c  # counter units per KiB actually moved by the copy
+            ent[counter] = round(k, 1)
+            ent[counter + "_copy"] = round(c, 1)
+            ent[counter + "_scale"] = round(scale, 4)
+            total += k * scale * 1024.0
+        if ent is not None:
+            ent["hbm_bytes_per_launch"] = int(round(total))
+            rec["workloads"][workload] = ent
+    os.makedirs(os.path.dirname(TRAFFIC_FILE), exist_ok=True)
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(rec, f, indent=1, sort_keys=True)
+        f.write("\n")
+    return rec
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -90,6 +153,10 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so a counter run can be scaled")
+    ap.add_argument("--traffic-from", metavar="DIR", default=None,
+                    help="no benchmark: read the rocprofv3 counter runs under DIR (pmc_FETCH_SIZE_<workload>/, "
+                         "pmc_WRITE_SIZE_<workload>/, each made with --copy-calibration) and write "
+                         "profiles/traffic.json, stamped with the digest of the kernel sources")
     args = ap.parse_args()
     args.gpt2_steps = args.steps if args.workload == "gpt2" and args.steps else 5
     args.gpt2_warmup = args.warmup if args.workload == "gpt2" and args.warmup is not None else 1
@@ -429,6 +496,11 @@ def bench_gpt2(args, torch, dev):
 
 def main():
     args = parse()
+    if args.traffic_from:
+        rec = traffic_record(args.traffic_from, args.seed)
+        print(json.dumps({"traffic_record": TRAFFIC_FILE, "workloads": sorted(rec["workloads"]),
+                          "csrc_sha256": rec["csrc_sha256"]}))
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the paged-attention path is single-GPU "
                  "(sequences and KV heads shard without communication); run with --gpus 1")

@@ -209,7 +209,11 @@ def test_decode_batch_beyond_the_lds_plan(gpu):
     coh = paged_ops.paged_decode(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens, d.max_context_len,
                                  cohort_size=16, cohort_shared_blocks=shared)
     torch.cuda.synchronize()
-    assert (coh.cpu().float() - out.float()).abs().max().item() <= 4e-3
+    _check(wl, coh.cpu())
+    # the two variants cut the rows at different tiles and merge in different orders: one step of
+    # bf16 at the value's magnitude
+    step = torch.maximum(torch.full_like(out.float(), 4e-3), out.float().abs() / 128)
+    assert ((coh.cpu().float() - out.float()).abs() - step).max().item() <= 0
 
 
 @pytest.mark.parametrize("hn,gn,dtype", [(8, 2, torch.bfloat16), (4, 4, torch.float16), (2, 1, torch.float32)])
