@@ -149,6 +149,8 @@ def parse():
     ap.add_argument("--cohort-size", type=int, default=0,
                     help="shared-prefix cohort size for decode (0 = the samples per prompt of the workload, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true",
+                    help="prefill: skip the 2 s measurement of the matrix rate the device sustains")
     ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU baseline time budget per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -399,6 +401,27 @@ def bench_prefill(args, torch, dev):
     rope_bytes = append_bytes + 2 * wl.query.numel() * es
     paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)  # leave the pool unrotated
 
+    # the matrix rate the device sustains once its clock has settled under load: a register-only
+    # MFMA loop on every SIMD, launched back to back for over a second, the last launches timed
+    sustained = None
+    if not args.no_mfma_probe:
+        sink = torch.zeros(16, dtype=torch.float32, device=dev)
+        iters = 20000  # about 6 ms per launch
+        t_end = time.perf_counter() + 1.5
+        probe_flops = 0
+        while time.perf_counter() < t_end:
+            for _ in range(10):
+                probe_flops = paged_ops.mfma_probe(iters, sink)
+            torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+        for a, b in ev:
+            a.record()
+            paged_ops.mfma_probe(iters, sink)
+            b.record()
+        torch.cuda.synchronize()
+        probe_ms = statistics.mean(a.elapsed_time(b) for a, b in ev)
+        sustained = probe_flops / (probe_ms * 1e-3) / 1e12
+
     result = {
         "metric": "paged_prefill_mfma_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "prefill_tokens_per_s_per_layer": round(n_tok / (ms_per_step * 1e-3), 1),
@@ -420,6 +443,15 @@ def bench_prefill(args, torch, dev):
     }
     if stale:
         result["roofline"]["traffic_stale"] = True
+    if sustained is not None:
+        # not the roofline's peak (that is the vendor's figure): what a bare MFMA loop reaches on
+        # this box, and the kernel's rate as a fraction of it
+        result["roofline"]["sustained_mfma"] = {
+            "value": round(sustained, 1), "unit": "TFLOP/s",
+            "what": "independent v_mfma_f32_32x32x16_bf16, register operands, one wave per SIMD, after 1.5 s of "
+                    "back-to-back launches (ic_mfma_probe)",
+            "frac_of_peak": round(sustained / MFMA_BF16_PEAK_TFLOPS, 4),
+            "kernel_frac_of_sustained": round(tflops / sustained, 4)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "kind": "port",
                                   "sample": f"all {len(wl.chunk_lens)} sequences of the batch, all heads, median of "

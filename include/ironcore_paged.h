@@ -72,6 +72,17 @@ int ic_version(void);
 const char *ic_error_string(int code);
 
 /*
+ * Diagnostic, no counterpart in the reference: launches a loop of `iters` x 16
+ * independent v_mfma_f32_32x32x16_bf16 per wave, one wave per SIMD on every
+ * CU, operands in registers (no memory, LDS or vector work), and returns the
+ * launch's flop count (negative: IC_ERR_*).  Timed over a second or more of
+ * back-to-back launches it gives the matrix rate the device sustains once its
+ * clock has settled under load, which bench.py reports beside the nominal
+ * 2.5 PFLOP/s.  sink: 4 bytes of device memory, never written in practice.
+ */
+int64_t ic_mfma_probe(int iters, void *sink, void *stream);
+
+/*
  * KV append: copy the K/V rows a transformer layer produced for n_tokens new
  * tokens into their cache slots, bit for bit.  Replaces nothing in the
  * reference (which recomputes K/V for the whole sequence every step,

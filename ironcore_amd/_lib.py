@@ -21,6 +21,7 @@ IC_DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 SIGNATURES = {
     "ic_version": (c_int, []),
     "ic_error_string": (c_char_p, [c_int]),
+    "ic_mfma_probe": (c_int64, [c_int, c_void_p, c_void_p]),
     "ic_kv_append": (c_int, [
         c_void_p, c_void_p, c_int64,            # k_new, v_new, new_stride_token
         c_void_p, c_void_p,                     # k_pool, v_pool

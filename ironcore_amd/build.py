@@ -20,7 +20,8 @@ LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libironcore_paged.so"
 OBJ_DIR = PKG / "build" / "obj"
 
-SOURCES = ["ic_api.hip", "kv_append.hip", "rope_kv_append.hip", "paged_decode.hip", "paged_decode_mfma.hip", "paged_prefill.hip"]
+SOURCES = ["ic_api.hip", "kv_append.hip", "rope_kv_append.hip", "paged_decode.hip", "paged_decode_mfma.hip", "paged_prefill.hip",
+           "mfma_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -203,6 +203,13 @@ extern "C" {
 
 int ic_version(void) { return 100; }
 
+int64_t ic_mfma_probe(int iters, void *sink, void *stream) {
+  if (sink == nullptr) return IC_ERR_NULL_POINTER;
+  if (iters < 1 || iters > (1 << 24)) return IC_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(sink) & 3) != 0) return IC_ERR_ALIGNMENT;
+  return ic::launch_mfma_probe(iters, sink, static_cast<hipStream_t>(stream));
+}
+
 const char *ic_error_string(int code) {
   switch (code) {
     case IC_OK: return "ok";

@@ -180,4 +180,7 @@ inline DecodeWorkspace decode_workspace(int n_seqs, int hn, int gn, int hd, int 
 // Compute units of the current device (cached per device ordinal).
 int device_cu_count();
 
+// Launches the matrix-rate probe (mfma_probe.hip); returns the launch's flop count or a negative IC_ERR_*.
+int64_t launch_mfma_probe(int iters, void *sink, hipStream_t stream);
+
 }  // namespace ic

@@ -58,6 +58,20 @@ class _Workspace:
 _workspace = _Workspace()
 
 
+def mfma_probe(iters: int, sink: torch.Tensor) -> int:
+    """Launch the matrix-rate probe (``iters`` x 16 register-only
+    v_mfma_f32_32x32x16_bf16 per wave, one wave per SIMD on every CU) on the
+    current stream and return the launch's flop count.  A diagnostic for the
+    benchmark; ``sink`` is any fp32 tensor on the GPU."""
+    lib = _lib.load()
+    dev = _require_gpu(sink)
+    with torch.cuda.device(dev):
+        rc = lib.ic_mfma_probe(int(iters), sink.data_ptr(), _lib.current_stream_ptr(dev))
+    if rc < 0:
+        _lib.check("ic_mfma_probe", int(rc))
+    return int(rc)
+
+
 def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
               slot_mapping: torch.Tensor) -> None:
     """Copy rows ``k_new[t]``, ``v_new[t]`` (``[n, gn, hd]``) into pool slot

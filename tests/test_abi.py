@@ -39,6 +39,13 @@ def test_version_and_error_strings():
     assert lib.ic_error_string(-99) == b"unknown error code"
 
 
+def test_mfma_probe_rejects_bad_arguments():
+    lib = _lib.load()
+    assert lib.ic_mfma_probe(100, None, None) == -1      # no sink
+    assert lib.ic_mfma_probe(0, 1 << 12, None) == -2     # no iterations
+    assert lib.ic_mfma_probe(100, (1 << 12) + 2, None) == -6
+
+
 def test_workspace_bytes():
     lib = _lib.load()
     assert lib.ic_paged_decode_workspace_bytes(0, 32, 32, 128) == 0
