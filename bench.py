@@ -149,6 +149,9 @@ def parse():
     ap.add_argument("--cohort-size", type=int, default=0,
                     help="shared-prefix cohort size for decode (0 = the samples per prompt of the workload, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="prefill: replace q, K and V by zeros (same kernel, same instructions, same bytes; shows "
+                         "how much of the launch time is the clock the device holds under toggling operands)")
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="prefill: skip the 2 s measurement of the matrix rate the device sustains")
     ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU baseline time budget per workload")
@@ -333,6 +336,9 @@ def bench_prefill(args, torch, dev):
     from ironcore_amd import paged_ops, workloads
     from oracle import paged as oracle_paged
     wl = workloads.llama7b_chunked_prefill(device=dev, seed=args.seed)
+    if args.zero_operands:
+        for t in (wl.query, wl.k_new, wl.v_new, wl.k_pool, wl.v_pool):
+            t.zero_()
     out = torch.empty(wl.query.shape[0], wl.hn * wl.hd, dtype=wl.query.dtype, device=dev)
 
     def step(i, ev):
@@ -427,7 +433,9 @@ def bench_prefill(args, torch, dev):
         "unit": "TFLOP/s", "prefill_tokens_per_s_per_layer": round(n_tok / (ms_per_step * 1e-3), 1),
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16",
+        "data": "synthetic, all-zero operands (a clock probe, not the benchmark workload)" if args.zero_operands
+                else "synthetic",
         "config": {"workload": wl.name, "n_seqs": len(wl.chunk_lens), "chunk": wl.max_chunk_len,
                    "sum_prefix": sum(wl.prefix_lens), "q_heads": wl.hn, "kv_heads": wl.gn,
                    "head_dim": wl.hd, "block_size": wl.block_size,
