@@ -393,31 +393,33 @@ __global__ __launch_bounds__(kReduceThreads) void paged_decode_reduce_kernel(con
     const int d = (o - g * QPH) * 4;
     float m_run = kNegInf, l_run = 0.f;
     float4 a_run = make_float4(0.f, 0.f, 0.f, 0.f);
+    // the partials of both sources as one list, fetched UB at a time: all loads of a batch are
+    // independent and in flight together, whichever source they come from
+    const int64_t n0 = w_hi[0] - w_lo[0] + 1, n_all = n0 + (w_hi[1] - w_lo[1] + 1);
+    for (int64_t ib = 0; ib < n_all; ib += UB) {
+      float2 ml[UB];
+      float4 av[UB];
 #pragma unroll
-    for (int src = 0; src < 2; ++src) {
-      for (int64_t wb = w_lo[src]; wb <= w_hi[src]; wb += UB) {
-        float2 ml[UB];
-        float4 av[UB];
+      for (int u = 0; u < UB; ++u) {
+        const int64_t i = ib + u < n_all ? ib + u : n_all - 1;
+        const int src = i < n0 ? 0 : 1;
+        const int64_t w = src == 0 ? w_lo[0] + i : w_lo[1] + (i - n0);
+        const int64_t slot = ((w + slot0[src]) * mul[src] + add[src]) * COLS + col0[src] + g;
+        ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
+        av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
+      }
 #pragma unroll
-        for (int u = 0; u < UB; ++u) {  // independent loads, all in flight together
-          const int64_t w = wb + u <= w_hi[src] ? wb + u : w_hi[src];
-          const int64_t slot = ((w + slot0[src]) * mul[src] + add[src]) * COLS + col0[src] + g;
-          ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
-          av[u] = *reinterpret_cast<const float4 *>(p.part_acc + slot * HD + d);
-        }
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          if (wb + u > w_hi[src] || ml[u].x == kNegInf) continue;
-          const float m_new = fmaxf(m_run, ml[u].x);
-          const float keep = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
-          const float wt = __builtin_amdgcn_exp2f(ml[u].x - m_new);
-          l_run = __builtin_fmaf(ml[u].y, wt, l_run * keep);
-          a_run.x = __builtin_fmaf(av[u].x, wt, a_run.x * keep);
-          a_run.y = __builtin_fmaf(av[u].y, wt, a_run.y * keep);
-          a_run.z = __builtin_fmaf(av[u].z, wt, a_run.z * keep);
-          a_run.w = __builtin_fmaf(av[u].w, wt, a_run.w * keep);
-          m_run = m_new;
-        }
+      for (int u = 0; u < UB; ++u) {
+        if (ib + u >= n_all || ml[u].x == kNegInf) continue;
+        const float m_new = fmaxf(m_run, ml[u].x);
+        const float keep = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float wt = __builtin_amdgcn_exp2f(ml[u].x - m_new);
+        l_run = __builtin_fmaf(ml[u].y, wt, l_run * keep);
+        a_run.x = __builtin_fmaf(av[u].x, wt, a_run.x * keep);
+        a_run.y = __builtin_fmaf(av[u].y, wt, a_run.y * keep);
+        a_run.z = __builtin_fmaf(av[u].z, wt, a_run.z * keep);
+        a_run.w = __builtin_fmaf(av[u].w, wt, a_run.w * keep);
+        m_run = m_new;
       }
     }
     const float inv = 1.f / l_run;
