@@ -48,7 +48,8 @@ namespace decode {
 namespace {
 
 constexpr float kLazyMaxSlack = 5.0f;  // log2 units
-constexpr int kLongRowTokens = 1024;     // longest context from which one workgroup per CU is launched
+constexpr int kLongRowTokens = 1024;      // longest context from which one workgroup per CU is launched
+constexpr int kVeryLongRowTokens = 4096;  // ... and from which one CU in eight is left out
 
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
@@ -531,8 +532,15 @@ bool launch_variant(DecodeKP &kp, size_t lds_bytes, hipStream_t stream) {
   // second workgroup pays: it hides the stalls of the row switches (query load, result write),
   // 7 % on 256 sequences of 64-512 tokens.  Cohorts keep both: their two phases overlap across
   // the workgroups of a CU.
-  if (!COOP && kp.cohort_size == 1 && kp.group >= 2 && kp.max_ctx >= kLongRowTokens && wgs > device_cu_count())
+  if (!COOP && kp.cohort_size == 1 && kp.group >= 2 && kp.max_ctx >= kLongRowTokens && wgs > device_cu_count()) {
     wgs = device_cu_count();
+    // Rows of several thousand tokens: seven workgroups per eight CUs (still a multiple of 8, so
+    // the XCD-major deal holds).  Measured +0.85 % at G = 8, +0.9 % at G = 4, +1.1 % at G = 2 with
+    // contexts of 1K-8K tokens (768 to 896 waves all the same, 1 024 slower: the requests of the
+    // last CUs only lengthen the queues of a memory system that is already full); with contexts
+    // up to 1K it loses 4-6 % (there the launch is short and every CU's share of it counts).
+    if (kp.max_ctx >= kVeryLongRowTokens) wgs = (wgs - wgs / 8) & ~7;
+  }
   if (wgs * NW > kp.max_waves) wgs = kp.max_waves / NW;
   kp.n_waves = wgs * NW;
   hipLaunchKernelGGL(kernel, dim3(wgs), dim3(NW * kWave), lds_bytes, stream, kp);
