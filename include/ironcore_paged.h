@@ -83,6 +83,16 @@ const char *ic_error_string(int code);
 int64_t ic_mfma_probe(int iters, void *sink, void *stream);
 
 /*
+ * Diagnostic, no counterpart in the reference: how many times the decode
+ * launcher has asked the HIP runtime for a kernel's occupancy in this process.
+ * The answers are kept per kernel variant and LDS size class (whole KiB), so
+ * the count stops growing once a serving loop has seen its batch-size classes;
+ * a launch whose answer is known makes no runtime query, which is what lets a
+ * stream capture on any host thread follow a warm-up on another.
+ */
+int64_t ic_decode_occupancy_queries(void);
+
+/*
  * KV append: copy the K/V rows a transformer layer produced for n_tokens new
  * tokens into their cache slots, bit for bit.  Replaces nothing in the
  * reference (which recomputes K/V for the whole sequence every step,
@@ -292,8 +302,9 @@ int ic_paged_prefill(void *out, int64_t out_stride_token,
  *
  *   mask    uint8; the byte of (sequence i, query head h, chunk row r, key j) is
  *           mask[i*mask_stride_seq + h*mask_stride_head + r*mask_stride_row + j],
- *           nonzero = visible.  A stride of 0 broadcasts over that index.  Rows
- *           must cover context_lens[i] keys.
+ *           nonzero = visible.  A stride of 0 broadcasts over that index.
+ *   mask_keys  keys every mask row covers (its extent along j): a key at or
+ *           beyond it is hidden, and no byte past it is read.
  * Hidden keys get the reference's FINITE fill value (attention.py:66): next to a
  * visible key they weigh nothing; a query row with no visible key returns the
  * plain average of V over its context, as the reference does.  A chunk may be
@@ -311,7 +322,7 @@ int ic_paged_prefill_masked(void *out, int64_t out_stride_token,
                             int64_t num_blocks, float scale,
                             const uint8_t *mask, int64_t mask_stride_seq,
                             int64_t mask_stride_head, int64_t mask_stride_row,
-                            int dtype, void *stream);
+                            int64_t mask_keys, int dtype, void *stream);
 
 /*
  * Paged decode under a key mask, fp32 only: ic_paged_decode where sequence i's

@@ -22,6 +22,7 @@ SIGNATURES = {
     "ic_version": (c_int, []),
     "ic_error_string": (c_char_p, [c_int]),
     "ic_mfma_probe": (c_int64, [c_int, c_void_p, c_void_p]),
+    "ic_decode_occupancy_queries": (c_int64, []),
     "ic_kv_append": (c_int, [
         c_void_p, c_void_p, c_int64,            # k_new, v_new, new_stride_token
         c_void_p, c_void_p,                     # k_pool, v_pool
@@ -86,7 +87,7 @@ SIGNATURES = {
         c_int, c_int, c_int, c_int,             # hn, gn, hd, block_size
         c_int64, c_float,                       # num_blocks, scale
         c_void_p, c_int64, c_int64, c_int64,    # mask, strides: seq, head, row
-        c_int, c_void_p]),                      # dtype, stream
+        c_int64, c_int, c_void_p]),             # mask_keys, dtype, stream
     "ic_paged_decode_masked": (c_int, [
         c_void_p, c_int64, c_void_p, c_int64,   # out, out_stride, q, q_stride
         c_void_p, c_void_p,                     # k_pool, v_pool

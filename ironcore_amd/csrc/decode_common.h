@@ -499,9 +499,11 @@ __device__ __forceinline__ int64_t window_tile_offset(const uint32_t *off_lo, co
 constexpr int kDecodeWavesPerWorkgroup = 4;
 
 // Launches the matrix-core decode main kernel (paged_decode_mfma.hip) when it
-// is built for this shape (16-bit dtype, hd 64 or 128, kp.gt <= 16 columns);
+// is built for this shape (16-bit dtype, hd 32, 64 or 128, kp.gt <= 16 columns);
 // returns false otherwise.  Sets kp.n_waves.
 bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream);
+// Runtime occupancy queries the matrix-core launcher has made in this process.
+long long decode_occupancy_queries();
 
 }  // namespace decode
 }  // namespace ic

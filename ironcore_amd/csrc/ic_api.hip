@@ -5,6 +5,12 @@
 #include "ic_internal.h"
 #include "../../include/ironcore_paged.h"
 
+namespace ic {
+namespace decode {
+long long decode_occupancy_queries();  // paged_decode_mfma.hip
+}
+}  // namespace ic
+
 // Device memory of the entry point that may not allocate (ic_paged_decode_static): the decode
 // workspace (row prefix sums and split-K partials) lives in this array instead of a buffer the
 // caller brings.  Every GPU the library runs on holds its own copy at its own address until the
@@ -137,8 +143,8 @@ int prefill_checked(void *out, int64_t out_stride_token, const void *q, int64_t 
                     int64_t block_table_stride, const int32_t *context_lens, const int32_t *cu_seqlens_q,
                     int n_seqs, int max_chunk_len, int hn, int gn, int hd, int block_size,
                     int64_t num_blocks, float scale, int causal, const uint8_t *mask,
-                    int64_t mask_stride_seq, int64_t mask_stride_head, int64_t mask_stride_row, int dtype,
-                    void *stream) {
+                    int64_t mask_stride_seq, int64_t mask_stride_head, int64_t mask_stride_row,
+                    int64_t mask_keys, int dtype, void *stream) {
   if (n_seqs < 0 || max_chunk_len < 0 || hn <= 0 || gn <= 0 || hn % gn != 0) return IC_ERR_BAD_SHAPE;
   if (!dtype_ok(dtype)) return IC_ERR_UNSUPPORTED;
   const int es = ic::elem_size(dtype);
@@ -177,6 +183,7 @@ int prefill_checked(void *out, int64_t out_stride_token, const void *q, int64_t 
   a.mask_stride_seq = mask_stride_seq;
   a.mask_stride_head = mask_stride_head;
   a.mask_stride_row = mask_stride_row;
+  a.mask_keys = mask_keys;
   return ic::launch_paged_prefill(a, static_cast<hipStream_t>(stream));
 }
 
@@ -201,7 +208,9 @@ int device_cu_count() {
 
 extern "C" {
 
-int ic_version(void) { return 100; }
+int ic_version(void) { return 200; }
+
+int64_t ic_decode_occupancy_queries(void) { return ic::decode::decode_occupancy_queries(); }
 
 int64_t ic_mfma_probe(int iters, void *sink, void *stream) {
   if (sink == nullptr) return IC_ERR_NULL_POINTER;
@@ -390,7 +399,7 @@ int ic_paged_prefill(void *out, int64_t out_stride_token, const void *q, int64_t
   return prefill_checked(out, out_stride_token, q, q_stride_token, k_pool, v_pool, pool_stride_block,
                          pool_stride_head, pool_stride_token, block_tables, block_table_stride,
                          context_lens, cu_seqlens_q, n_seqs, max_chunk_len, hn, gn, hd, block_size,
-                         num_blocks, scale, causal, nullptr, 0, 0, 0, dtype, stream);
+                         num_blocks, scale, causal, nullptr, 0, 0, 0, 0, dtype, stream);
 }
 
 int ic_paged_prefill_masked(void *out, int64_t out_stride_token, const void *q, int64_t q_stride_token,
@@ -401,14 +410,16 @@ int ic_paged_prefill_masked(void *out, int64_t out_stride_token, const void *q, 
                             int max_chunk_len, int hn, int gn, int hd, int block_size,
                             int64_t num_blocks, float scale, const uint8_t *mask,
                             int64_t mask_stride_seq, int64_t mask_stride_head, int64_t mask_stride_row,
-                            int dtype, void *stream) {
+                            int64_t mask_keys, int dtype, void *stream) {
   if (n_seqs > 0 && max_chunk_len > 0 && mask == nullptr) return IC_ERR_NULL_POINTER;
-  if (mask_stride_seq < 0 || mask_stride_head < 0 || mask_stride_row < 0) return IC_ERR_BAD_SHAPE;
+  if (mask_stride_seq < 0 || mask_stride_head < 0 || mask_stride_row < 0 || mask_keys < 0) return IC_ERR_BAD_SHAPE;
+  if (mask_stride_row != 0 && mask_stride_row < mask_keys) return IC_ERR_BAD_SHAPE;
+  if (n_seqs > 0 && max_chunk_len > 0 && mask_keys < 1) return IC_ERR_BAD_SHAPE;  // a mask row holds a byte at least
   return prefill_checked(out, out_stride_token, q, q_stride_token, k_pool, v_pool, pool_stride_block,
                          pool_stride_head, pool_stride_token, block_tables, block_table_stride,
                          context_lens, cu_seqlens_q, n_seqs, max_chunk_len, hn, gn, hd, block_size,
                          num_blocks, scale, 0, mask, mask_stride_seq, mask_stride_head, mask_stride_row,
-                         dtype, stream);
+                         mask_keys, dtype, stream);
 }
 
 int ic_paged_decode_masked(void *out, int64_t out_stride_seq, const void *q, int64_t q_stride_seq,

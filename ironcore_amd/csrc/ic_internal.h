@@ -102,6 +102,7 @@ struct PrefillArgs {
   int64_t mask_stride_seq = 0;
   int64_t mask_stride_head = 0;
   int64_t mask_stride_row = 0;
+  int64_t mask_keys = 0;  // keys a mask row covers; keys from there on are hidden
 };
 
 // Each returns IC_OK, IC_ERR_UNSUPPORTED (no kernel built for this

@@ -488,6 +488,7 @@ int launch_group(DecodeKP &kp, int dtype, hipStream_t stream) {
 template <class E>
 int launch_hd(DecodeKP &kp, int hd, int dtype, hipStream_t stream) {
   switch (hd) {
+    case 32: return launch_group<E, 32>(kp, dtype, stream);
     case 64: return launch_group<E, 64>(kp, dtype, stream);
     case 128: return launch_group<E, 128>(kp, dtype, stream);
     default: return IC_ERR_UNSUPPORTED;

@@ -37,6 +37,7 @@
 // Per tile and wave: hd/32 + hd/16 MFMAs, about 70 vector instructions and
 // 2 * hd/32 LDS accesses, whatever G is: about 0.6 us when the tile is in the
 // cache, which leaves the kernel bound by HBM for any pool that is not.
+#include <atomic>
 #include <type_traits>
 
 #include "decode_common.h"
@@ -46,6 +47,8 @@ namespace ic {
 namespace decode {
 
 namespace {
+
+std::atomic<long long> g_occupancy_queries{0};  // runtime occupancy queries made so far (a diagnostic)
 
 constexpr float kLazyMaxSlack = 5.0f;  // log2 units
 constexpr int kLongRowTokens = 1024;      // longest context from which one workgroup per CU is launched
@@ -106,6 +109,10 @@ __device__ __forceinline__ VChunk<2> load_v<2>(const void *p) {
   const uint2 v = *reinterpret_cast<const uint2 *>(p);
   return VChunk<2>{{v.x, v.y}};
 }
+template <>
+__device__ __forceinline__ VChunk<1> load_v<1>(const void *p) {
+  return VChunk<1>{{*reinterpret_cast<const uint32_t *>(p)}};
+}
 
 // With shared-prefix cohorts the kernel runs two phases (see DecodeKP); every
 // other workgroup takes them in the opposite order, so that the LDS-fed
@@ -130,7 +137,7 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
   constexpr int VW = VE / 2;   // dwords per V load
   constexpr int NT = 4;        // tokens per lane on the V side
   constexpr int SW = 4;
-  static_assert(sizeof(T) == 2 && BS == 16 && (VW == 2 || VW == 4), "tile shape");
+  static_assert(sizeof(T) == 2 && BS == 16 && (VW == 1 || VW == 2 || VW == 4), "tile shape");
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -303,16 +310,22 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
           for (int k = 0; k < VW; ++k)
             packed[k] = E::pack(acc[cb][2 * k][r] * inv, acc[cb][2 * k + 1][r] * inv);
           char *o = p.out + (seq * p.out_stride_seq + (int64_t)head * HD + n * VE) * ES;
-          if (VW == 4)
+          if constexpr (VW == 4)
             store16(o, Vec16{{packed[0], packed[1], packed[2 % VW], packed[3 % VW]}});
+          else if constexpr (VW == 2)
+            *reinterpret_cast<uint2 *>(o) = make_uint2(packed[0], packed[1 % VW]);
           else
-            *reinterpret_cast<uint2 *>(o) = make_uint2(packed[0], packed[1]);
+            *reinterpret_cast<uint32_t *>(o) = packed[0];
         } else {
           float *o = p.part_acc + (partial * COLS + col) * HD + n * VE;
+          if constexpr (VE >= 4) {
 #pragma unroll
-          for (int k = 0; k < VE / 4; ++k)
-            *reinterpret_cast<float4 *>(o + 4 * k) = make_float4(acc[cb][4 * k][r], acc[cb][4 * k + 1][r],
-                                                                 acc[cb][4 * k + 2][r], acc[cb][4 * k + 3][r]);
+            for (int k = 0; k < VE / 4; ++k)
+              *reinterpret_cast<float4 *>(o + 4 * k) = make_float4(acc[cb][4 * k][r], acc[cb][4 * k + 1][r],
+                                                                   acc[cb][4 * k + 2][r], acc[cb][4 * k + 3][r]);
+          } else {
+            *reinterpret_cast<float2 *>(o) = make_float2(acc[cb][0][r], acc[cb][1][r]);
+          }
         }
       }
       if (!whole_pair && kg == 0) {
@@ -457,8 +470,10 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
         for (int j = 0; j < NT * VW / 4; ++j) {
           if constexpr (VW == 4)
             dst[j * kWave] = Vec16{{va[j].w[0], va[j].w[1], va[j].w[2 % VW], va[j].w[3 % VW]}};
+          else if constexpr (VW == 2)
+            dst[j * kWave] = Vec16{{va[2 * j].w[0], va[2 * j].w[1 % VW], va[2 * j + 1].w[0], va[2 * j + 1].w[1 % VW]}};
           else
-            dst[j * kWave] = Vec16{{va[2 * j].w[0], va[2 * j].w[1], va[2 * j + 1].w[0], va[2 * j + 1].w[1]}};
+            dst[j * kWave] = Vec16{{va[0].w[0], va[1].w[0], va[2].w[0], va[3].w[0]}};
         }
       };
       auto get = [&](int slot) {
@@ -470,9 +485,12 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
           const Vec16 v = src[j * kWave];
           if constexpr (VW == 4) {
             vb[j] = VChunk<VW>{{v.w[0], v.w[1], v.w[2 % VW], v.w[3 % VW]}};
-          } else {
+          } else if constexpr (VW == 2) {
             vb[2 * j] = VChunk<VW>{{v.w[0], v.w[1]}};
             vb[2 * j + 1] = VChunk<VW>{{v.w[2], v.w[3]}};
+          } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) vb[t] = VChunk<VW>{{v.w[t]}};
           }
         }
       };
@@ -506,21 +524,28 @@ template <class E, int HD, int NW, bool PLAN, bool COOP>
 bool launch_variant(DecodeKP &kp, size_t lds_bytes, hipStream_t stream) {
   constexpr int BS = 16;
   auto kernel = paged_decode_mfma_kernel<E, HD, BS, NW, PLAN, COOP>;
-  constexpr size_t kMaxLds = (PLAN ? kPlanMaxInts * sizeof(int) : 0) + tiles_lds_bytes(HD, NW, COOP);
+  constexpr size_t kLdsGranule = 1024;
+  constexpr size_t kMaxLds =
+      ((PLAN ? kPlanMaxInts * sizeof(int) : 0) + tiles_lds_bytes(HD, NW, COOP) + kLdsGranule - 1) / kLdsGranule * kLdsGranule;
   static const bool ready = [&] {  // more than 64 KB of dynamic LDS has to be asked for
     return kMaxLds <= 64 * 1024 ||
            hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)kMaxLds) == hipSuccess;
   }();
   if (!ready) return false;
-  // workgroups one CU holds with this much LDS (remembered for the last size asked)
-  thread_local size_t seen_bytes = ~(size_t)0;
-  thread_local int per_cu = 1;
-  if (seen_bytes != lds_bytes) {
+  // Workgroups one CU holds with this much LDS.  The plan's share of LDS grows with the batch, so
+  // the request is rounded up to whole KiB and the runtime's answer kept per KiB count, for the
+  // whole process: a serving loop whose batch size changes from step to step asks once per size
+  // class, and a stream capture on any host thread finds the answers a warm-up on another left.
+  lds_bytes = (lds_bytes + kLdsGranule - 1) / kLdsGranule * kLdsGranule;
+  static std::atomic<int> per_cu_of[kMaxLds / kLdsGranule + 2];  // 0 = not asked yet
+  int per_cu = per_cu_of[lds_bytes / kLdsGranule].load(std::memory_order_relaxed);
+  if (per_cu == 0) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NW * kWave, lds_bytes) != hipSuccess || n < 1) n = 1;
+    g_occupancy_queries.fetch_add(1, std::memory_order_relaxed);
     per_cu = n;
-    seen_bytes = lds_bytes;
+    per_cu_of[lds_bytes / kLdsGranule].store(n, std::memory_order_relaxed);
   }
   int wgs = per_cu * device_cu_count();
   // Long rows: one workgroup per CU.  A wave keeps two tiles (16 KiB at head dim 128) in flight,
@@ -577,6 +602,7 @@ bool launch_one(DecodeKP &kp, hipStream_t stream) {
 template <class E>
 bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
   switch (hd) {
+    case 32: return launch_one<E, 32>(kp, stream);
     case 64: return launch_one<E, 64>(kp, stream);
     case 128: return launch_one<E, 128>(kp, stream);
     default: return false;
@@ -584,6 +610,8 @@ bool launch_hd(DecodeKP &kp, int hd, hipStream_t stream) {
 }
 
 }  // namespace
+
+long long decode_occupancy_queries() { return g_occupancy_queries.load(std::memory_order_relaxed); }
 
 bool launch_decode_mfma_main(DecodeKP &kp, int dtype, int hd, hipStream_t stream) {
   if (kp.gt < 1 || kp.gt > kCohortColumnsPerWave || (1 << kp.unit_shift) > kMaxCohortWaves) return false;

@@ -74,8 +74,9 @@ struct PrefillKP {
   int64_t stride_token;
   int64_t bt_stride;
   int64_t num_blocks;
-  int block_size;
+  int block_size;   // a multiple of 16 tokens
   int block_shift;  // log2(block_size) when it is a power of two, else -1
+  uint32_t block_magic;  // otherwise floor(2^32 / (block_size / 16)) + 1: n / (block_size / 16) == mulhi(n, magic)
   int group;        // query heads per KV head
   int gn;           // KV heads
   int n_units;      // n_seqs * gn
@@ -88,6 +89,7 @@ struct PrefillKP {
   int64_t mask_stride_seq;
   int64_t mask_stride_head;
   int64_t mask_stride_row;
+  int mask_keys;  // keys a mask row covers: keys from there on are hidden and never read
 };
 
 constexpr float kNegInf = -__builtin_huge_valf();
@@ -146,7 +148,7 @@ constexpr int kBM = kPrefillWaves * 32;   // query rows per workgroup
 constexpr int kStageBuffers = 4;          // LDS buffers per pool: a tile is fetched three tiles ahead
 
 // SINGLE: every sequence is one pool block (a dense [b, sk, gn, hd] tensor
-// viewed as a pool); otherwise blocks are a power of two >= 16 tokens long.
+// viewed as a pool); otherwise blocks are a multiple of 16 tokens long.
 // MASK: visibility comes from a byte mask instead of the causal rule; every
 // query row walks all L keys and a chunk may be longer than its context.
 template <class M, int HD, bool SINGLE, bool MASK>
@@ -160,19 +162,20 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   constexpr int NST = 16 / WR;         // loads (16-byte pieces) per lane and staged tile
   constexpr int ROWB = HD * 2;         // bytes of one token row; LDS tiles are unpadded [token][dim]
   constexpr int NB = kStageBuffers;    // LDS buffers per pool
-  static_assert(kBN == 64 && 16 % WR == 0 && (CPR == 8 || CPR == 16), "tile staging shape");
+  static_assert(kBN == 64 && 16 % WR == 0 && (CPR == 4 || CPR == 8 || CPR == 16), "tile staging shape");
 
   // A tile reaches LDS straight from memory (global_load_lds: no registers, no LDS write
   // instruction), 1 KiB per wave and load, lane l's 16 bytes at byte 16*l of that KiB.  Rows are
   // therefore unpadded, and what keeps the operand reads free of bank conflicts is a swizzle:
   // 16-byte chunk c of tile row r lives in slot c ^ swz(r) of its row (the lane that fills a slot
   // simply fetches the chunk that belongs there).  K (read as whole 16-byte chunks, 16 rows per
-  // access): swz = r % 16 (head dim 128), (r / 2) % 8 (head dim 64).  V (read by the transposing
-  // 8-byte reads, 4 rows x 64 bytes per access): swz = 4 * (r % 4), resp. 4 * ((r / 2) % 2).
+  // access): swz = r % 16 (head dim 128), (r / 2) % 8 (head dim 64), (r / 4) % 4 (head dim 32).
+  // V (read by the transposing 8-byte reads, 4 rows x 64 bytes per access): swz = 4 * (r % 4),
+  // resp. 4 * ((r / 2) % 2); none at head dim 32, where a row is one 64-byte group.
   __shared__ __attribute__((aligned(1024))) char s_k[NB][kBN * ROWB];
   __shared__ __attribute__((aligned(1024))) char s_v[NB][kBN * ROWB];
-  auto swz_k = [](int r) { return CPR == 16 ? (r & 15) : ((r >> 1) & 7); };
-  auto swz_v = [](int r) { return CPR == 16 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2); };
+  auto swz_k = [](int r) { return CPR == 16 ? (r & 15) : CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
+  auto swz_v = [](int r) { return CPR == 16 ? ((r & 3) << 2) : CPR == 8 ? (((r >> 1) & 1) << 2) : 0; };
 
   // XCD-aware placement.  Workgroups are dealt to the 8 XCDs round-robin by
   // their linear id, and each XCD has its own L2.  All workgroups that read
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // ---- tile staging: memory -> LDS ---------------------------------------------------
   // A wave stages one 16-row group of every tile (group wave & 3) of ONE pool:
   // the waves of side 0 stage K, those of side 1 stage V.  Pool blocks are a
-  // power of two >= 16 rows long (or the sequence is a single block), so a
+  // multiple of 16 rows long (or the sequence is a single block), so a
   // group lies inside one block: one table entry and one base address per wave
   // and tile, scalar work, and a lane only adds fixed offsets.  Nothing here is
   // conditional: a tile index past the sweep is clamped to the last tile, a
@@ -283,7 +286,12 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int rsub = lane / CPR;  // row within the rows one load covers
   const char *stage_pool = side == 0 ? p.k_pool : p.v_pool;
   const int64_t head_off = (int64_t)kvh * p.stride_head;
-  const int last_blk = SINGLE ? 0 : (L - 1) >> p.block_shift;
+  // pool block of a row that starts a 16-row group (wave-uniform, scalar unit): a shift for
+  // power-of-two blocks, else a multiplication by the reciprocal the host prepared
+  auto block_of = [&](int row) {
+    return p.block_shift >= 0 ? row >> p.block_shift : (int)__umulhi((uint32_t)row >> 4, p.block_magic);
+  };
+  const int last_blk = SINGLE ? 0 : block_of((L - 1) & ~15);
   typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
   const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
   // byte offset, from the group's first row, of the chunk lane l fetches with load i: row
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   auto clamp_tile = [&](int tile) { return tile < n_tiles ? tile : n_tiles - 1; };
   auto lookup = [&](int tile, int32_t &ent) {
     const int first = clamp_tile(tile) * kBN + 16 * grp;  // this wave's first row of the tile
-    int blk = SINGLE ? 0 : first >> p.block_shift;
+    int blk = SINGLE ? 0 : block_of(first);
     blk = blk < last_blk ? blk : last_blk;
     ent = table_row[blk];
   };
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
                      :: "s"(dst + i * WR * ROWB), "v"(src) : "memory", "m0");
       }
     } else {
-      const int rem = first & (p.block_size - 1);
+      const int rem = first - block_of(first) * p.block_size;
       const char *base = stage_pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2;
 #pragma unroll
       for (int i = 0; i < NST; ++i)
@@ -382,7 +390,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     // scheduler issues them two at a time, right before the MFMAs that need
     // them, and every pair waits out an LDS round trip (+2.5 % on the kernel;
     // the other product already gets its reads eight ahead).
-    constexpr int kAhead = 6;
+    constexpr int kAhead = TB * KS < 6 ? TB * KS : 6;
     __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
     for (int i = 0; i < TB * KS - kAhead; ++i) {
@@ -408,12 +416,25 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
     if constexpr (MASK) {  // keys the caller's mask hides from this lane's query row
       const uint8_t *mrow = p.mask + (int64_t)seq * p.mask_stride_seq + (int64_t)h * p.mask_stride_head +
                             (int64_t)qrow * p.mask_stride_row;
+      // Every byte is fetched unconditionally, from an index clamped into the part of the row
+      // that exists and counts (keys below both the context length and the mask's extent), so
+      // the 32 loads of a tile are independent and in flight together; a key past the mask's
+      // extent is hidden whatever the byte fetched in its place says.
+      const int last = (limit < p.mask_keys - 1 ? limit : p.mask_keys - 1);
+      uint8_t seen[TB][16];
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
-          const bool hidden = tok <= limit && mrow[tok] == 0;
+          seen[tb][i] = mrow[tok < last ? tok : last];
+        }
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int tok = tok_base + tb * 32 + 8 * (i / 4) + (i & 3);
+          const bool hidden = (tok <= limit) & ((tok >= p.mask_keys) | (seen[tb][i] == 0));
           s[tb][i] = hidden ? kHiddenScore : s[tb][i];
         }
     }
@@ -602,6 +623,9 @@ int launch_hd(PrefillKP kp, const PrefillArgs &a, hipStream_t stream) {
   if (wgs > 0x7fffffff) return IC_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)wgs);
   switch (a.hd) {
+    case 32:
+      hipLaunchKernelGGL((paged_prefill_kernel<M, 32, SINGLE, MASK>), grid, dim3(kPrefillThreads), 0, stream, kp);
+      break;
     case 64:
       hipLaunchKernelGGL((paged_prefill_kernel<M, 64, SINGLE, MASK>), grid, dim3(kPrefillThreads), 0, stream, kp);
       break;
@@ -620,7 +644,7 @@ int launch_mode(const PrefillKP &kp, const PrefillArgs &a, hipStream_t stream) {
   const bool masked = a.mask != nullptr;
   if (a.block_table_stride == 1)
     return masked ? launch_hd<M, true, true>(kp, a, stream) : launch_hd<M, true, false>(kp, a, stream);
-  if (kp.block_shift < 4) return IC_ERR_UNSUPPORTED;  // power-of-two blocks of >= 16 tokens
+  if (kp.block_size < 16 || kp.block_size % 16 != 0) return IC_ERR_UNSUPPORTED;  // whole 16-token groups
   return masked ? launch_hd<M, false, true>(kp, a, stream) : launch_hd<M, false, false>(kp, a, stream);
 }
 
@@ -646,6 +670,14 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   kp.block_shift = -1;
   for (int s = 0; s < 31; ++s)
     if ((1 << s) == a.pool.block_size) kp.block_shift = s;
+  kp.block_magic = 0;
+  if (kp.block_shift < 0 && a.pool.block_size >= 16) {
+    // exact for token rows below 2^40 / block_size; longer tables are refused
+    kp.block_magic = (uint32_t)((1ull << 32) / (uint32_t)(a.pool.block_size / 16)) + 1u;
+    if (a.block_table_stride > 1 &&
+        a.block_table_stride * (int64_t)a.pool.block_size >= ((int64_t)1 << 40) / a.pool.block_size)
+      return IC_ERR_UNSUPPORTED;
+  }
   kp.group = a.hn / a.gn;
   kp.gn = a.gn;
   kp.n_units = a.n_seqs * a.gn;
@@ -656,6 +688,7 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   kp.mask_stride_seq = a.mask_stride_seq;
   kp.mask_stride_head = a.mask_stride_head;
   kp.mask_stride_row = a.mask_stride_row;
+  kp.mask_keys = a.mask_keys > 0x7fffffff ? 0x7fffffff : (int)a.mask_keys;
   if ((int64_t)a.max_chunk_len >= (int64_t)65535 * 128 || a.hn > 65535 || a.n_seqs > 65535)
     return IC_ERR_UNSUPPORTED;
   switch (a.dtype) {

@@ -28,14 +28,29 @@ from dataclasses import dataclass
 from typing import Optional
 
 import torch
+import torch.nn.functional as F
 from torch import nn
 
 from .. import paged_ops
 from .module import BaseModule, get_model_dtype
 
 
-# attention_mask tensor -> what _classify_mask found for it: id -> (weak reference, (version, shapes), kind, bytes)
+# attention_mask tensor -> what _classify_mask found for it: id -> (weak reference, (version, shapes), kind, bytes).
+# An entry goes when its mask tensor dies (the weak reference's callback) and when more than
+# _MASK_CLASSES_MAX masks are alive at once (oldest first): the byte copy of a general mask is as
+# large as the mask, and a model that builds a new document mask per batch must not pile them up.
 _MASK_CLASSES: dict = {}
+_MASK_CLASSES_MAX = 4
+
+
+def _mask_version(mask):
+    """The tensor's in-place edit counter, or None for a tensor that keeps none
+    (one created under torch.inference_mode()): such a mask is classified on
+    every call, since an edit to it could not be noticed."""
+    try:
+        return mask._version
+    except RuntimeError:
+        return None
 
 
 @dataclass
@@ -124,8 +139,9 @@ class Attention(BaseModule):
         pays once per forward pass, not once per layer."""
         if attention_mask is None:
             return "none", None
-        hit = _MASK_CLASSES.get(id(attention_mask))
-        if hit is not None and hit[0]() is attention_mask and hit[1] == (attention_mask._version, b, sq, sk, hn):
+        version = _mask_version(attention_mask)
+        hit = _MASK_CLASSES.get(id(attention_mask)) if version is not None else None
+        if hit is not None and hit[0]() is attention_mask and hit[1] == (version, b, sq, sk, hn):
             return hit[2], hit[3]
         m = attention_mask
         while m.dim() < 4:
@@ -144,11 +160,16 @@ class Attention(BaseModule):
             kind, data = "causal", None
         else:
             kind, data = "general", visible.to(torch.uint8).contiguous()
-        if len(_MASK_CLASSES) > 64:
-            for key in [k for k, v in _MASK_CLASSES.items() if v[0]() is None]:
-                del _MASK_CLASSES[key]
-        _MASK_CLASSES[id(attention_mask)] = (weakref.ref(attention_mask), (attention_mask._version, b, sq, sk, hn),
-                                             kind, data)
+        if version is not None:
+            key = id(attention_mask)
+            _MASK_CLASSES.pop(key, None)
+            while len(_MASK_CLASSES) >= _MASK_CLASSES_MAX:
+                del _MASK_CLASSES[next(iter(_MASK_CLASSES))]
+
+            def forget(ref, key=key):
+                if key in _MASK_CLASSES and _MASK_CLASSES[key][0] is ref:
+                    del _MASK_CLASSES[key]
+            _MASK_CLASSES[key] = (weakref.ref(attention_mask, forget), (version, b, sq, sk, hn), kind, data)
         return kind, data
 
     # ------------------------------------------------------------------ forward
@@ -172,6 +193,22 @@ class Attention(BaseModule):
         sk, gn = key.shape[1], key.shape[2]
         kind, mask = self._classify_mask(attention_mask, b, sq, sk, hn)
         causal = kind == "causal"
+        if hd not in paged_ops.SUPPORTED_HEAD_DIMS:
+            # The reference takes any d_model // heads (attention.py:51).  Zero columns appended
+            # to query, key and value change no score (the scale stays 1/sqrt(hd)) and add zero
+            # output columns, so a head dimension between the built ones runs on the next one up.
+            wide = next((w for w in paged_ops.SUPPORTED_HEAD_DIMS if w > hd), None)
+            if wide is None:
+                raise ValueError(f"head dimension {hd}: the attention kernels are built for "
+                                 f"{paged_ops.SUPPORTED_HEAD_DIMS} and pad smaller ones up to the next of them")
+            pad = (0, wide - hd)
+            padded = self._dense_on_kernel_width(F.pad(query, pad), F.pad(key, pad), F.pad(value, pad), causal, mask)
+            return padded.view(b, sq, hn, wide)[..., :hd].reshape(b, sq, hn * hd)
+        return self._dense_on_kernel_width(query, key, value, causal, mask)
+
+    def _dense_on_kernel_width(self, query, key, value, causal, mask):
+        b, sq, hn, hd = query.shape
+        sk, gn = key.shape[1], key.shape[2]
         if query.dtype == torch.float32:
             return self._dense_fp32(query, key, value, causal, mask)
         key, value = key.contiguous(), value.contiguous()

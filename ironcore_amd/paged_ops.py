@@ -28,6 +28,16 @@ def _require_gpu(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
+# Head dimensions the attention kernels are built for (the append kernels take any multiple of
+# 16 bytes).  The layer's dense call pads smaller ones up to the next entry.
+SUPPORTED_HEAD_DIMS = (32, 64, 128)
+
+
+def _require_head_dim(hd: int) -> None:
+    if hd not in SUPPORTED_HEAD_DIMS:
+        raise ValueError(f"the attention kernels are built for head dimensions {SUPPORTED_HEAD_DIMS}, got {hd}")
+
+
 def _pool_strides(k_pool: torch.Tensor, v_pool: torch.Tensor):
     if k_pool.dim() != 4 or k_pool.shape != v_pool.shape or k_pool.stride() != v_pool.stride():
         raise ValueError("k_pool and v_pool must be [num_blocks, gn, block_size, hd] with equal strides")
@@ -183,6 +193,7 @@ def paged_decode(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
     if query.dim() != 3 or query.shape[2] != hd:
         raise ValueError(f"query must be [b, hn, {hd}], got {tuple(query.shape)}")
+    _require_head_dim(hd)
     if query.dtype != k_pool.dtype:
         raise TypeError("query and pools must share a dtype")
     b, hn, _ = query.shape
@@ -262,6 +273,7 @@ def paged_decode_static(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
     if query.dim() != 3 or query.shape[2] != hd or query.stride(2) != 1 or query.stride(1) != hd:
         raise ValueError(f"query must be [b, hn, {hd}] with contiguous heads")
+    _require_head_dim(hd)
     if query.dtype != k_pool.dtype:
         raise TypeError("query and pools must share a dtype")
     b, hn, _ = query.shape
@@ -323,15 +335,17 @@ def paged_prefill(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
     ``cu_seqlens_q[i]:cu_seqlens_q[i+1]``); the chunk's K/V are already in the
     pool and ``context_lens[i]`` counts prefix + chunk.  -> ``[n_tokens, hn*hd]``.
 
-    ``mask`` (uint8 ``[1 or n_seqs, 1 or hn, >= max_chunk_len, >= max context]``,
+    ``mask`` (uint8 ``[1 or n_seqs, 1 or hn, >= max_chunk_len, keys]``,
     last dimension contiguous) replaces the causal rule: byte (i, h, r, j) == 0
-    hides key j from row r of chunk i (head h).  Hidden keys get the
+    hides key j from row r of chunk i (head h); a key past the mask's last
+    dimension is hidden too (nothing is read beyond it).  Hidden keys get the
     reference's finite fill value: a row that sees nothing averages V."""
     lib = _lib.load()
     dev = _require_gpu(query, k_pool, v_pool, block_tables, context_lens, cu_seqlens_q)
     nb, gn, bs, hd, sb, sh, st = _pool_strides(k_pool, v_pool)
     if query.dim() != 3 or query.shape[2] != hd:
         raise ValueError(f"query must be [n_tokens, hn, {hd}], got {tuple(query.shape)}")
+    _require_head_dim(hd)
     if query.dtype != k_pool.dtype:
         raise TypeError("query and pools must share a dtype")
     n_tokens, hn, _ = query.shape
@@ -369,7 +383,7 @@ def paged_prefill(query: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
                                              mask.data_ptr(),
                                              mask.stride(0) if mask.shape[0] > 1 else 0,
                                              mask.stride(1) if mask.shape[1] > 1 else 0, mask.stride(2),
-                                             _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
+                                             mask.shape[3], _lib.dtype_code(query.dtype), _lib.current_stream_ptr(dev))
         _lib.check("ic_paged_prefill_masked", rc)
         return out
     with torch.cuda.device(dev):

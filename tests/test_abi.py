@@ -115,6 +115,43 @@ def test_prefill_argument_errors():
     assert call(q=(1 << 13) + 8) == -6
 
 
+def test_masked_entry_points_argument_errors():
+    """ic_paged_prefill_masked and ic_paged_decode_masked: a missing mask, negative
+    strides, a mask row shorter than the keys it is said to cover, a key mask
+    narrower than max_context_len and element types the kernels do not take are
+    all refused on the host."""
+    lib = _lib.load()
+
+    def prefill(mask=1 << 19, s_seq=0, s_head=0, s_row=4608, keys=4608, dtype=0, n=4, q=1 << 13):
+        return lib.ic_paged_prefill_masked(1 << 12, 4096, q, 4096, 1 << 14, 1 << 15, 65536, 2048, 128, 1 << 16, 300,
+                                           1 << 17, 1 << 18, n, 512, 32, 32, 128, 16, 1000, 0.0884, mask, s_seq,
+                                           s_head, s_row, keys, dtype, None)
+    assert prefill(n=0, mask=None, q=None) == 0
+    assert prefill(mask=None) == -1
+    assert prefill(s_seq=-1) == -2
+    assert prefill(s_head=-8) == -2
+    assert prefill(s_row=-4608) == -2
+    assert prefill(keys=-1) == -2
+    assert prefill(s_row=100, keys=4608) == -2      # rows overlap the keys they are said to cover
+    assert prefill(dtype=9) == -3
+
+    def decode(key_mask=1 << 19, s_seq=4096, s_head=0, dtype=2, n=64, st=128, sb=32 * 16 * 128):
+        a = DECODE_OK
+        return lib.ic_paged_decode_masked(a["out"], a["out_stride"], a["q"], a["q_stride"], a["kp"], a["vp"], sb,
+                                          a["sh"], st, a["bt"], a["bt_stride"], a["cl"], n, a["hn"], a["gn"],
+                                          a["hd"], a["bs"], a["nb"], a["max_ctx"], a["scale"], 0, key_mask, s_seq,
+                                          s_head, a["ws"], a["ws_bytes"], dtype, None)
+    assert decode(n=0) == 0
+    assert decode(key_mask=None) == -1
+    assert decode(s_seq=4095) == -2                  # narrower than max_context_len
+    assert decode(s_head=-1) == -2
+    assert decode(dtype=0) == -3 and decode(dtype=1) == -3   # 16-bit calls use ic_paged_prefill_masked
+
+
+def test_occupancy_query_counter_starts_at_zero_without_a_gpu():
+    assert _lib.load().ic_decode_occupancy_queries() >= 0
+
+
 def test_python_wrapper_rejects_cpu_tensors():
     import torch
     from ironcore_amd import paged_ops

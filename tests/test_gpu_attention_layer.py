@@ -51,6 +51,46 @@ def test_dense_call_matches_reference_arithmetic(gpu, dtype, precision, tol, hn,
     assert (got.cpu().float() - want.float()).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("dtype,precision,tol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "fp32", 1e-4)])
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_reference_head_dimension_sweep(gpu, dtype, precision, tol, hd):
+    """The reference's own sweep (tests/test_attention.py:352-379): 8 heads,
+    d_model = 8 * head_dim for head_dim in {32, 64, 128}, batch 2, 64 tokens, the
+    float lower-triangular mask expanded to [b, 1, s, s] (its
+    create_causal_mask, :105-109); there the call only has to return the right
+    shape, here the values are held to the oracle as well."""
+    b, s, hn = 2, 64, 8
+    q, k, v = _qkv(b, s, s, hn, hn, hd, dtype, seed=hd)
+    mask = torch.tril(torch.ones(s, s)).unsqueeze(0).unsqueeze(0).expand(b, -1, -1, -1)
+    want = dense_attention(q, k, v, mask)
+    attn = Attention(_cfg(hn, hn, hd, precision)).to(gpu).eval()
+    assert attn.head_dimension == hd
+    got = attn(q.to(gpu), k.to(gpu), v.to(gpu), mask.to(gpu))
+    torch.cuda.synchronize()
+    assert got.shape == (b, s, hn * hd)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype,precision,tol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "fp32", 1e-4)])
+@pytest.mark.parametrize("hd", [8, 20, 48, 96, 120])
+def test_dense_call_with_head_dimensions_between_the_built_ones(gpu, dtype, precision, tol, hd):
+    """The reference takes any d_model // heads (attention.py:51): the dense call
+    pads the head dimension with zero columns up to the next one a kernel is
+    built for, which changes no score and no output column.  Larger than the
+    largest raises, naming them."""
+    b, sq, sk, hn, gn = 2, 50, 90, 6, 3
+    q, k, v = _qkv(b, sq, sk, hn, gn, hd, dtype, seed=hd)
+    mask = causal_offset_mask(sq, sk)
+    _dense_vs_oracle(gpu, q, k, v, mask, precision, tol, f"hd {hd}")
+
+
+def test_dense_call_with_a_head_dimension_beyond_the_largest_kernel(gpu):
+    q, k, v = _qkv(1, 4, 4, 2, 2, 256, torch.bfloat16, seed=0)
+    attn = Attention(_cfg(2, 2, 256, "bf16")).to(gpu).eval()
+    with pytest.raises(ValueError, match=r"\(32, 64, 128\)"):
+        attn(q.to(gpu), k.to(gpu), v.to(gpu))
+
+
 def test_dense_call_with_shorter_query(gpu):
     q, k, v = _qkv(2, 5, 40, 4, 4, 128, torch.bfloat16, seed=1)
     mask = causal_offset_mask(5, 40)
@@ -171,8 +211,9 @@ def test_mask_is_classified_once_per_tensor(gpu):
 
 
 @pytest.mark.parametrize("dtype,precision,tol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "fp32", 1e-4)])
-def test_paged_prefill_then_decode_through_the_layer(gpu, dtype, precision, tol):
-    hn, gn, hd, b = 8, 4, 64, 3
+@pytest.mark.parametrize("hd", [32, 64])
+def test_paged_prefill_then_decode_through_the_layer(gpu, dtype, precision, tol, hd):
+    hn, gn, b = 8, 4, 3
     attn = Attention(_cfg(hn, gn, hd, precision)).to(gpu).eval()
     cache = PagedKVCache(1, 32, 16, gn, hd, dtype, gpu)
     ids = [cache.add_sequence() for _ in range(b)]

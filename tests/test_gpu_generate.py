@@ -138,6 +138,34 @@ def test_multiple_choice_scoring_matches_oracle(gpu, positional):
     assert scoring.pick_endings(prompts, got.tolist(), labels) == scoring.pick_endings(prompts, want.tolist(), labels)
 
 
+def test_scoring_batch_of_eighty_sequences_bf16(gpu):
+    """A scoring batch wider than one wave's lanes (80 sequences: the prefill
+    kernel then finds a workgroup's sequence by direct lookup instead of the
+    in-wave ranking).  bf16 model; losses against the fp32 CPU oracle on the
+    same weights within bf16's reach, against the same sequences scored 16 at a
+    time (the ranked path) tightly, and the same endings picked."""
+    import torch.nn.functional as F
+    from ironcore_amd import scoring
+    cfg = _small("bf16", 2)
+    torch.manual_seed(4)
+    model = generation.LanguageModel(cfg, vocab_size=1000)
+    w = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    g = torch.Generator().manual_seed(9)
+    tokens = torch.randint(0, 1000, (80, 33), generator=g)
+    tokens[::5, 25:] = 999
+    logits = oracle_gpt2.forward_full(w, _dims(cfg), tokens[:, :-1])
+    want = torch.stack([F.cross_entropy(logits[i], tokens[i, 1:]) for i in range(80)])
+    model = model.to(gpu).to(torch.bfloat16).eval()
+    got = scoring.per_sample_losses(model, tokens.to(gpu))
+    by16 = torch.cat([scoring.per_sample_losses(model, tokens[i:i + 16].to(gpu)) for i in range(0, 80, 16)])
+    assert (got - by16).abs().max().item() < 2e-2
+    assert (got - want).abs().max().item() < 6e-2
+    prompts = [i // 4 for i in range(80)]
+    labels = [1 if i % 4 == 1 else 0 for i in range(80)]
+    picked, picked16 = scoring.pick_endings(prompts, got.tolist(), labels), scoring.pick_endings(prompts, by16.tolist(), labels)
+    assert abs(picked["score"] - picked16["score"]) <= 5.0   # 20 questions: at most one near-tie may flip
+
+
 @pytest.mark.parametrize("precision,positional,groups", [("fp32", "absolute", 4), ("fp32", "rope", 2),
                                                          ("bf16", "absolute", 1), ("bf16", "rope", 4)])
 def test_graph_replay_generate_equals_the_step_by_step_loop(gpu, precision, positional, groups):

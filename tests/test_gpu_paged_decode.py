@@ -40,10 +40,35 @@ def test_decode_group_sizes_bf16(gpu, hn, gn):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("hd", [32, 64, 128])
 def test_decode_dtypes_head_dims(gpu, dtype, hd):
     wl = workloads.make_decode_workload(5, 8, 4, hd, 1, 900, dtype=dtype, seed=hd)
     _check(wl, _run(wl, gpu))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hn,gn", [(8, 8), (8, 1), (7, 1), (24, 2)])
+def test_decode_head_dim_32_group_sizes(gpu, dtype, hn, gn):
+    """Head dimension 32 (the smallest the reference's own sweep uses,
+    tests/test_attention.py:352-379) over MHA, MQA, an odd group and a group
+    wider than one wave's columns; contexts long enough for split-K partials."""
+    wl = workloads.make_decode_workload(7, hn, gn, 32, 1, 2600, dtype=dtype, seed=hn * 10 + gn)
+    out = _run(wl, gpu)
+    _check(wl, out)
+    one = _run(wl, gpu, min_chunk_tokens=1 << 20)          # one wave walks everything: no partials
+    assert (out.float() - one.float()).abs().max().item() <= (4e-3 if dtype != torch.float32 else 1e-5)
+
+
+def test_unsupported_head_dims_are_named_before_the_c_call(gpu):
+    """A head dimension without a kernel is refused in Python, with the list of
+    those that have one, not by an error code from the library."""
+    kp = torch.zeros(2, 1, 16, 96, dtype=torch.bfloat16, device=gpu)
+    tables, lens = torch.zeros(1, 1, dtype=torch.int32, device=gpu), torch.ones(1, dtype=torch.int32, device=gpu)
+    q = torch.zeros(1, 1, 96, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(ValueError, match=r"\(32, 64, 128\)"):
+        paged_ops.paged_decode(q, kp, kp, tables, lens, 1)
+    with pytest.raises(ValueError, match=r"\(32, 64, 128\)"):
+        paged_ops.paged_prefill(q, kp, kp, tables, lens, torch.tensor([0, 1], dtype=torch.int32, device=gpu), 1)
 
 
 @pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 511, 512, 513, 1024, 1025])

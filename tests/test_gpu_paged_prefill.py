@@ -45,10 +45,52 @@ def test_prefill_prefix_chunk_shapes(gpu, prefix, chunk):
 
 
 @pytest.mark.parametrize("hn,gn", [(8, 8), (8, 2), (8, 1), (28, 4)])
-@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("hd", [32, 64, 128])
 def test_prefill_gqa_and_head_dims(gpu, hn, gn, hd):
     wl = workloads.make_prefill_workload(3, hn, gn, hd, 0, 200, 1, 150, seed=hn + gn + hd)
     _check(wl, gpu)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("prefix,chunk,block", [(0, 300, 16), (700, 130, 16), (45, 257, 64)])
+def test_prefill_head_dim_32(gpu, dtype, prefix, chunk, block):
+    """Head dimension 32: several K/V tiles, two query tiles, both block sizes."""
+    wl = workloads.make_prefill_workload(3, 6, 2, 32, prefix, prefix + 40, 1, chunk, block_size=block, dtype=dtype,
+                                         seed=prefix + chunk)
+    _check(wl, gpu)
+
+
+@pytest.mark.parametrize("n_seqs", [64, 65, 130])
+def test_prefill_many_sequences(gpu, n_seqs):
+    """Batches at and beyond one sequence per lane: up to 64 sequences the
+    kernel ranks them by context length inside a wave (64 exactly fills it),
+    beyond that a workgroup looks its sequence up directly.  Short ragged
+    chunks (some empty) behind short prefixes, with equal context lengths among
+    them so that the ranking's tie rule decides."""
+    wl = workloads.make_prefill_workload(n_seqs, 4, 2, 64, 0, 100, 0, 40, seed=n_seqs)
+    lens = wl.context_lens.tolist()
+    assert len(set(lens)) < len(lens), "the draw should contain equal context lengths"
+    assert 0 in wl.chunk_lens
+    _check(wl, gpu)
+
+
+@pytest.mark.parametrize("block", [48, 80, 112])
+def test_prefill_block_sizes_that_are_no_power_of_two(gpu, block):
+    """Any multiple of 16 tokens is a block size (the decode kernel and the
+    cache take them too): prefill, then a decode step over the same pools."""
+    wl = workloads.make_prefill_workload(3, 8, 2, 128, 0, 500, 1, 300, block_size=block, seed=block)
+    _check(wl, gpu)
+    d = wl.to(gpu)
+    paged_ops.kv_append(d.k_new, d.v_new, d.k_pool, d.v_pool, d.slot_mapping)
+    last = (d.cu_seqlens_q[1:] - 1).long()
+    keep = [i for i, c in enumerate(wl.chunk_lens) if c > 0]
+    q = d.query.index_select(0, last[keep])
+    dec = paged_ops.paged_decode(q, d.k_pool, d.v_pool, d.block_tables[keep], d.context_lens[keep].contiguous(),
+                                 int(wl.context_lens.max()))
+    pre = paged_ops.paged_prefill(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens, d.cu_seqlens_q,
+                                  d.max_chunk_len)
+    torch.cuda.synchronize()
+    assert (dec.float() - pre.index_select(0, last[keep]).float()).abs().max().item() <= 4e-3
 
 
 def test_prefill_fp16(gpu):

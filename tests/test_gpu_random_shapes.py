@@ -26,9 +26,9 @@ def _f64(*tensors):
     return [t.double() for t in tensors]
 
 
-def _draw_decode(rng):
+def _draw_decode(rng, dims=(64, 128)):
     hn, gn = HEADS[rng.integers(len(HEADS))]
-    hd = int(rng.choice([64, 128]))
+    hd = int(rng.choice(dims))
     dtype = DTYPES[rng.integers(len(DTYPES))]
     block = int(rng.choice([16, 16, 32, 64]))
     batch = int(rng.choice([1, 2, 3, 7, 16, 33, 90]))
@@ -39,8 +39,16 @@ def _draw_decode(rng):
 
 @pytest.mark.parametrize("case", range(80))
 def test_random_decode(gpu, case):
-    rng = np.random.default_rng(1000 + case)
-    hn, gn, hd, dtype, block, batch, lo, hi = _draw_decode(rng)
+    _random_decode(gpu, case, np.random.default_rng(1000 + case))
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_random_decode_head_dim_32(gpu, case):
+    _random_decode(gpu, 4000 + case, np.random.default_rng(4000 + case), dims=(32,))
+
+
+def _random_decode(gpu, case, rng, dims=(64, 128)):
+    hn, gn, hd, dtype, block, batch, lo, hi = _draw_decode(rng, dims)
     min_chunk = int(rng.choice([16, 64, 512, 1 << 20]))
     print(f"decode case {case}: hn {hn} gn {gn} hd {hd} {dtype} block {block} batch {batch} ctx [{lo}, {hi}] "
           f"min_chunk_tokens {min_chunk}", flush=True)
@@ -57,9 +65,17 @@ def test_random_decode(gpu, case):
 
 @pytest.mark.parametrize("case", range(48))
 def test_random_cohorts(gpu, case):
-    rng = np.random.default_rng(2000 + case)
+    _random_cohorts(gpu, case, np.random.default_rng(2000 + case))
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_random_cohorts_head_dim_32(gpu, case):
+    _random_cohorts(gpu, 5000 + case, np.random.default_rng(5000 + case), dims=(32,))
+
+
+def _random_cohorts(gpu, case, rng, dims=(64, 128)):
     hn, gn = HEADS[rng.integers(len(HEADS))]
-    hd = int(rng.choice([64, 128]))
+    hd = int(rng.choice(dims))
     dtype = [torch.bfloat16, torch.float16][rng.integers(2)]
     block = int(rng.choice([16, 16, 32, 64]))
     group = hn // gn
@@ -92,9 +108,17 @@ def test_random_cohorts(gpu, case):
 
 @pytest.mark.parametrize("case", range(48))
 def test_random_prefill(gpu, case):
-    rng = np.random.default_rng(3000 + case)
+    _random_prefill(gpu, case, np.random.default_rng(3000 + case))
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_random_prefill_head_dim_32(gpu, case):
+    _random_prefill(gpu, 6000 + case, np.random.default_rng(6000 + case), dims=(32,))
+
+
+def _random_prefill(gpu, case, rng, dims=(64, 128)):
     hn, gn = HEADS[rng.integers(len(HEADS))]
-    hd = int(rng.choice([64, 128]))
+    hd = int(rng.choice(dims))
     dtype = [torch.bfloat16, torch.bfloat16, torch.float16][rng.integers(3)]
     block = int(rng.choice([16, 16, 32, 64]))
     n_seqs = int(rng.choice([1, 2, 5, 9]))

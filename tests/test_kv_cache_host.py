@@ -256,3 +256,46 @@ def test_attention_refuses_inputs_that_require_grad():
     with torch.no_grad():                            # not recording: passes the check (and then needs a GPU)
         with pytest.raises(RuntimeError, match="GPU only"):
             attn(q, k, v)
+
+
+def test_masks_built_under_inference_mode_and_the_mask_cache_stays_small():
+    """A tensor created under torch.inference_mode() keeps no version counter:
+    the layer classifies such a mask on every call instead of failing on it (the
+    call then goes on to the device check).  And the per-tensor cache of
+    classified masks holds a few live masks at most and lets go of a mask's
+    byte copy when the mask tensor dies."""
+    import gc
+    import pytest
+    import torch
+    from ironcore_amd import config as ic_config
+    from ironcore_amd.layers import Attention
+    from ironcore_amd.layers import attention as attention_module
+    cfg = ic_config.MainConfig(model=ic_config.ModelConfig(d_model=128, num_attention_heads=2,
+                                                           num_attention_groups=2, head_dim=64, dropout_attn=0.0,
+                                                           precision="bf16"),
+                               trainer=ic_config.TrainerConfig(use_flash_attn=False))
+    attn = Attention(cfg).eval()
+    with torch.inference_mode():
+        q = torch.randn(1, 4, 2, 64)
+        mask = torch.tril(torch.ones(1, 1, 4, 4))
+        assert attn._classify_mask(mask, 1, 4, 4, 2) == ("causal", None)
+        mask[0, 0, 3, 0] = 0
+        kind, data = attn._classify_mask(mask, 1, 4, 4, 2)       # the edit is seen: nothing was cached
+        assert kind == "general" and data[0, 0, 3].tolist() == [0, 1, 1, 1]
+        with pytest.raises(RuntimeError, match="GPU only"):
+            attn(q, q, q, mask)
+    attention_module._MASK_CLASSES.clear()
+    masks = []
+    for i in range(10):
+        m = torch.ones(1, 1, 4, 4)
+        m[0, 0, 0, 1 + i % 3] = 0
+        assert attn._classify_mask(m, 1, 4, 4, 2)[0] == "general"
+        masks.append(m)
+        assert len(attention_module._MASK_CLASSES) <= attention_module._MASK_CLASSES_MAX
+    kept = len(attention_module._MASK_CLASSES)
+    assert kept == attention_module._MASK_CLASSES_MAX
+    again = attn._classify_mask(masks[-1], 1, 4, 4, 2)            # a cached answer: the same byte tensor
+    assert again[1] is attention_module._MASK_CLASSES[id(masks[-1])][3]
+    del masks, m, again
+    gc.collect()
+    assert len(attention_module._MASK_CLASSES) == 0
