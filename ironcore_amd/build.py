@@ -21,7 +21,7 @@ LIB_PATH = LIB_DIR / "libironcore_paged.so"
 OBJ_DIR = PKG / "build" / "obj"
 
 SOURCES = ["ic_api.hip", "kv_append.hip", "rope_kv_append.hip", "paged_decode.hip", "paged_decode_mfma.hip", "paged_prefill.hip",
-           "mfma_probe.hip"]
+           "paged_prefill_f32.hip", "mfma_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -61,7 +61,8 @@ def _hipcc() -> str:
 # VGPRs: the softmax rescales them with VALU instructions, and the AGPR form
 # costs a register copy each way per tile.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
-PER_SOURCE_FLAGS = {"paged_prefill.hip": _VGPR_FORM, "paged_decode_mfma.hip": _VGPR_FORM}
+PER_SOURCE_FLAGS = {"paged_prefill.hip": _VGPR_FORM, "paged_prefill_f32.hip": _VGPR_FORM,
+                    "paged_decode_mfma.hip": _VGPR_FORM}
 
 
 def _compile(src: str, extra: list[str]) -> Path:

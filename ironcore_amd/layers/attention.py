@@ -18,8 +18,11 @@ appends the new ``key``/``value`` rows to the layer's block pool and attends
 against the cache (decode kernel for sq == 1, chunked-prefill kernel
 otherwise).  Without ``kv_cache`` the call is the reference's dense call; it
 runs on the same chunked-prefill kernel by viewing ``key``/``value`` as a pool
-with one block per sequence.  Every path runs the hand-written HIP kernels;
-there is no torch fallback.
+with one block per sequence.  bf16 and fp16 tensors take the 16-bit matrix-core
+kernels, fp32 tensors (what the reference's own contract tests pass,
+tests/test_attention.py:143-161) the fp32 ones, with every product, sum and
+probability in fp32.  Every path runs the hand-written HIP kernels; there is
+no torch fallback.
 """
 from __future__ import annotations
 
@@ -209,8 +212,6 @@ class Attention(BaseModule):
     def _dense_on_kernel_width(self, query, key, value, causal, mask):
         b, sq, hn, hd = query.shape
         sk, gn = key.shape[1], key.shape[2]
-        if query.dtype == torch.float32:
-            return self._dense_fp32(query, key, value, causal, mask)
         key, value = key.contiguous(), value.contiguous()
         # one pool block per sequence: [b, gn, sk, hd] view of the [b, sk, gn, hd] rows
         k_pool, v_pool = key.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)
@@ -228,36 +229,11 @@ class Attention(BaseModule):
         return zeros."""
         b, sq, hn, hd = query.shape
         packed = query.reshape(b * sq, hn, hd).index_select(0, rows)
-        if query.dtype == torch.float32:
-            got = _ragged_rows_fp32(packed, k_pool, v_pool, meta, scale)
-        else:
-            got = paged_ops.paged_prefill(packed, k_pool, v_pool, meta.block_tables, meta.context_lens,
-                                          meta.cu_seqlens_q, meta.max_chunk_len, causal=True, scale=scale)
+        got = paged_ops.paged_prefill(packed, k_pool, v_pool, meta.block_tables, meta.context_lens,
+                                      meta.cu_seqlens_q, meta.max_chunk_len, causal=True, scale=scale)
         out = query.new_zeros(b * sq, hn * hd)
         out.index_copy_(0, rows, got)
         return out.view(b, sq, hn * hd)
-
-    def _dense_fp32(self, query, key, value, causal, mask=None):
-        """fp32 has no MFMA path: every query row runs as one decode-kernel
-        sequence over the keys it may see (fp32 loads, fp32 arithmetic); a
-        general mask travels as one key-mask row per query row.  K and V are
-        streamed once per query ROW, so this costs sq times the traffic of the
-        16-bit kernel: it is there for exactness at small sizes, not speed."""
-        b, sq, hn, hd = query.shape
-        sk, gn = key.shape[1], key.shape[2]
-        dev = query.device
-        # The decode kernel loads whole 16-token tiles: give every sequence a
-        # block padded to a multiple of 16 rows (rows past sk are never visible).
-        sk16 = (sk + 15) // 16 * 16
-        k_rows = key.new_zeros(b, sk16, gn, hd)
-        v_rows = value.new_zeros(b, sk16, gn, hd)
-        k_rows[:, :sk] = key
-        v_rows[:, :sk] = value
-        k_pool, v_pool = k_rows.permute(0, 2, 1, 3), v_rows.permute(0, 2, 1, 3)
-        return _fp32_rows_via_decode(query, k_pool, v_pool,
-                                     torch.arange(b, dtype=torch.int32, device=dev).unsqueeze(1),
-                                     torch.full((b,), sk, dtype=torch.int32, device=dev), sk, causal,
-                                     1.0 / self.scale_factor, mask)
 
     def _paged(self, query, key, value, kv_cache, meta, rotary_pos_emb=None):
         if meta is None:
@@ -289,51 +265,9 @@ class Attention(BaseModule):
                                          cohort_size=cohort,
                                          cohort_shared_blocks=meta.cohort_shared_blocks if cohort > 1 else None)
             return out.view(b, 1, hn * hd)
-        if query.dtype == torch.float32:
-            return _fp32_rows_via_decode(query, k_pool, v_pool, meta.block_tables, meta.context_lens,
-                                         meta.max_context_len, True, scale)
         cu = meta.cu_seqlens_q
         if cu is None:
             cu = torch.arange(0, (b + 1) * sq, sq, dtype=torch.int32, device=query.device)
         out = paged_ops.paged_prefill(query.reshape(b * sq, hn, hd), k_pool, v_pool, meta.block_tables,
                                       meta.context_lens, cu, sq, causal=True, scale=scale)
         return out.view(b, sq, hn * hd)
-
-
-def _ragged_rows_fp32(query_rows, k_pool, v_pool, meta, scale):
-    """fp32 chunks of unequal length: every existing query row as one
-    decode-kernel sequence over the keys it may see."""
-    cu = meta.cu_seqlens_q.long()
-    counts = cu[1:] - cu[:-1]
-    seq_of_row = torch.repeat_interleave(torch.arange(counts.numel(), device=cu.device), counts)
-    back = (cu[1:].index_select(0, seq_of_row) - 1) - torch.arange(seq_of_row.numel(), device=cu.device)
-    ctx = (meta.context_lens.long().index_select(0, seq_of_row) - back).to(torch.int32)
-    tables = meta.block_tables.index_select(0, seq_of_row)
-    return paged_ops.paged_decode(query_rows, k_pool, v_pool, tables, ctx, meta.max_context_len, scale=scale)
-
-
-def _fp32_rows_via_decode(query, k_pool, v_pool, block_tables, context_lens, max_context_len, causal, scale,
-                          mask=None):
-    """Chunk attention in fp32: query row r of sequence i becomes one
-    decode-kernel sequence with context_lens[i] - (sq - 1 - r) visible tokens
-    (all of them when not causal), sharing sequence i's block-table row.
-    ``mask`` (uint8 [1 or b, 1 or hn, sq, sk]) hides keys per query row."""
-    b, sq, hn, hd = query.shape
-    dev = query.device
-    rows = torch.arange(b, device=dev).repeat_interleave(sq)
-    tables = block_tables.index_select(0, rows)
-    if mask is not None:
-        mh, sk = mask.shape[1], mask.shape[3]
-        key_mask = mask.expand(b, mh, sq, sk).permute(0, 2, 1, 3).reshape(b * sq, mh, sk).contiguous()
-        ctx = context_lens.index_select(0, rows).contiguous()
-        out = paged_ops.paged_decode(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx,
-                                     max_context_len, scale=scale, key_mask=key_mask)
-        return out.view(b, sq, hn * hd)
-    if causal:
-        back = (sq - 1 - torch.arange(sq, device=dev, dtype=torch.int32)).repeat(b)
-        ctx = (context_lens.index_select(0, rows) - back).to(torch.int32)
-    else:
-        ctx = context_lens.index_select(0, rows).contiguous()
-    out = paged_ops.paged_decode(query.reshape(b * sq, hn, hd), k_pool, v_pool, tables, ctx,
-                                 max_context_len, scale=scale)
-    return out.view(b, sq, hn * hd)

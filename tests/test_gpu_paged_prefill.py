@@ -1,6 +1,7 @@
-"""Chunked prefill (MFMA kernel) through the C ABI against the CPU oracle: the
-reference's dense attention with the offset causal mask on the gathered rows.
-Tolerance: max-abs 2e-2 (bf16/fp16), the bound the target states."""
+"""Chunked prefill (the 16-bit and the fp32 matrix-core kernels) through the C
+ABI against the CPU oracle: the reference's dense attention with the offset
+causal mask on the gathered rows.  Tolerance: max-abs 2e-2 (bf16/fp16), the
+bound the target states; 1e-4 for fp32 pools."""
 import pytest
 import torch
 
@@ -9,6 +10,7 @@ from oracle import paged as oracle_paged
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
+FP32_TOL = 1e-4
 
 
 def _run(wl, gpu, causal=True):
@@ -26,14 +28,17 @@ def _oracle(wl):
     return oracle_paged.paged_prefill(wl.query, kp, vp, wl.block_tables, wl.context_lens, wl.cu_seqlens_q), kp, vp
 
 
-def _check(wl, gpu):
+def _check(wl, gpu, tol=None):
     out, d = _run(wl, gpu)
     ref, kp, vp = _oracle(wl)
-    assert torch.equal(d.k_pool.cpu().view(torch.int16), kp.view(torch.int16)), "append not bit-exact"
-    assert torch.equal(d.v_pool.cpu().view(torch.int16), vp.view(torch.int16)), "append not bit-exact"
+    fp32 = wl.query.dtype == torch.float32
+    bits = torch.int32 if fp32 else torch.int16
+    assert torch.equal(d.k_pool.cpu().view(bits), kp.view(bits)), "append not bit-exact"
+    assert torch.equal(d.v_pool.cpu().view(bits), vp.view(bits)), "append not bit-exact"
     assert torch.isfinite(out.float()).all()
     diff = (out.float() - ref.float()).abs().max().item()
-    assert diff <= TOL, f"max|diff| {diff}"
+    tol = tol or (FP32_TOL if fp32 else TOL)
+    assert diff <= tol, f"max|diff| {diff}"
     return diff
 
 
@@ -91,6 +96,73 @@ def test_prefill_block_sizes_that_are_no_power_of_two(gpu, block):
                                   d.max_chunk_len)
     torch.cuda.synchronize()
     assert (dec.float() - pre.index_select(0, last[keep]).float()).abs().max().item() <= 4e-3
+
+
+@pytest.mark.parametrize("prefix,chunk", [(0, 1), (0, 17), (0, 128), (5, 64), (100, 33), (64, 129), (300, 200),
+                                          (1000, 256), (63, 65), (31, 300)])
+def test_prefill_fp32_prefix_chunk_shapes(gpu, prefix, chunk):
+    """fp32 pools: 32-token K/V tiles, 128-row query tiles, every product and sum in fp32."""
+    wl = workloads.make_prefill_workload(2, 4, 4, 128, prefix, prefix, chunk, chunk, dtype=torch.float32,
+                                         seed=prefix + chunk)
+    _check(wl, gpu)
+
+
+@pytest.mark.parametrize("hn,gn", [(8, 8), (8, 2), (6, 1), (28, 4)])
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_prefill_fp32_gqa_and_head_dims(gpu, hn, gn, hd):
+    wl = workloads.make_prefill_workload(3, hn, gn, hd, 0, 200, 1, 150, dtype=torch.float32, seed=hn + gn + hd)
+    _check(wl, gpu)
+
+
+@pytest.mark.parametrize("block", [16, 48, 64, 80])
+def test_prefill_fp32_block_sizes_ragged_batch(gpu, block):
+    """Ragged chunks (one of them empty) over several block sizes, among them ones that are no
+    power of two."""
+    wl = workloads.make_prefill_workload(6, 4, 2, 64, 0, 300, 0, 200, block_size=block, dtype=torch.float32,
+                                         seed=block)
+    _check(wl, gpu)
+
+
+def test_prefill_fp32_many_sequences_and_garbage_in_unused_slots(gpu):
+    wl = workloads.make_prefill_workload(70, 2, 1, 32, 0, 60, 0, 50, dtype=torch.float32, seed=70)
+    for i in range(70):
+        ctx = int(wl.context_lens[i])
+        if ctx % 16:
+            last = wl.block_tables[i, (ctx - 1) // 16].long()
+            wl.k_pool[last, :, ctx % 16:, :] = float("nan")
+            wl.v_pool[last, :, ctx % 16:, :] = float("nan")
+    _check(wl, gpu)
+
+
+def test_prefill_fp32_non_causal_and_decode_agreement(gpu):
+    """Without the causal rule every row sees the whole context; and the last row of a causal chunk
+    equals a decode step over the same pools (two kernels, one answer)."""
+    from oracle.dense_attention import dense_attention
+    wl = workloads.make_prefill_workload(3, 6, 2, 128, 20, 400, 30, 70, dtype=torch.float32, seed=23)
+    out, d = _run(wl, gpu, causal=False)
+    kp, vp = d.k_pool.cpu(), d.v_pool.cpu()
+    refs = []
+    for i in range(3):
+        lo, hi = int(wl.cu_seqlens_q[i]), int(wl.cu_seqlens_q[i + 1])
+        ctx = int(wl.context_lens[i])
+        k = oracle_paged.gather_kv(kp, wl.block_tables[i], ctx)
+        v = oracle_paged.gather_kv(vp, wl.block_tables[i], ctx)
+        refs.append(dense_attention(wl.query[lo:hi][None], k, v, None)[0])
+    assert (out - torch.cat(refs)).abs().max().item() <= FP32_TOL
+    causal = paged_ops.paged_prefill(d.query, d.k_pool, d.v_pool, d.block_tables, d.context_lens, d.cu_seqlens_q,
+                                     d.max_chunk_len)
+    last = (d.cu_seqlens_q[1:] - 1).long()
+    dec = paged_ops.paged_decode(d.query.index_select(0, last), d.k_pool, d.v_pool, d.block_tables, d.context_lens,
+                                 int(wl.context_lens.max()))
+    torch.cuda.synchronize()
+    assert (dec - causal.index_select(0, last)).abs().max().item() <= 2e-5
+
+
+def test_prefill_fp32_llama7b_chunk(gpu):
+    """One sequence at the benchmark's dims in fp32: 32 heads of 128, a 512-token chunk behind
+    2 048 cached tokens (what ran as 512 decode rows per head before this kernel existed)."""
+    wl = workloads.make_prefill_workload(1, 32, 32, 128, 2048, 2048, 512, 512, dtype=torch.float32, seed=1)
+    _check(wl, gpu)
 
 
 def test_prefill_fp16(gpu):
