@@ -146,6 +146,8 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
 
   const int64_t wave_id = (int64_t)xcd_major_workgroup() * NW + wave;
   const bool cohorts = p.cohort_size > 1;
+  typedef const __attribute__((address_space(4))) int32_t *ScalarPtr;  // read through the scalar cache
+  const ScalarPtr ctx_lens = (ScalarPtr)(unsigned long long)p.context_lens;
   extern __shared__ int plan_mem[];
   PlanLds plan;
   if constexpr (PLAN) {
@@ -354,7 +356,9 @@ void paged_decode_mfma_kernel(const DecodeKP p) {
     int ctx_here = 0x7fffffff;
     const int tok0 = (c.first + c.blk) * BS;
     if (c.blk == c.nb - 1) {
-      int ctx = __builtin_amdgcn_readfirstlane(p.context_lens[c.tseq]);
+      // (a scalar load: it waits on the scalar counter only, where a vector load would have to
+      // be waited for with everything before it, the prefetched tile included)
+      int ctx = ctx_lens[c.tseq];
       ctx = ctx < p.max_ctx ? ctx : p.max_ctx;
       if (tok0 + BS > ctx) {
         ctx_here = ctx;
