@@ -116,11 +116,20 @@ def test_random_prefill_head_dim_32(gpu, case):
     _random_prefill(gpu, 6000 + case, np.random.default_rng(6000 + case), dims=(32,))
 
 
-def _random_prefill(gpu, case, rng, dims=(64, 128)):
+@pytest.mark.parametrize("case", range(32))
+def test_random_prefill_fp32(gpu, case):
+    """fp32 pools (the fp32 matrix-instruction kernel), all three head dims, block sizes that are no
+    power of two among them."""
+    _random_prefill(gpu, 7000 + case, np.random.default_rng(7000 + case), dims=(32, 64, 128),
+                    dtypes=(torch.float32,), blocks=(16, 16, 32, 48, 64, 80))
+
+
+def _random_prefill(gpu, case, rng, dims=(64, 128), dtypes=(torch.bfloat16, torch.bfloat16, torch.float16),
+                    blocks=(16, 16, 32, 64)):
     hn, gn = HEADS[rng.integers(len(HEADS))]
     hd = int(rng.choice(dims))
-    dtype = [torch.bfloat16, torch.bfloat16, torch.float16][rng.integers(3)]
-    block = int(rng.choice([16, 16, 32, 64]))
+    dtype = dtypes[rng.integers(len(dtypes))]
+    block = int(rng.choice(blocks))
     n_seqs = int(rng.choice([1, 2, 5, 9]))
     p_hi = int(rng.choice([0, 30, 300, 900]))
     c_hi = int(rng.choice([1, 40, 260, 520]))
@@ -143,8 +152,9 @@ def _random_prefill(gpu, case, rng, dims=(64, 128)):
     torch.cuda.synchronize()
     kp, vp = wl.k_pool.clone(), wl.v_pool.clone()
     oracle_paged.kv_append(kp, vp, wl.k_new, wl.v_new, wl.slot_mapping)
-    assert torch.equal(d.k_pool.cpu().view(torch.int16), kp.view(torch.int16)), "append not bit-exact"
-    assert torch.equal(d.v_pool.cpu().view(torch.int16), vp.view(torch.int16)), "append not bit-exact"
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    assert torch.equal(d.k_pool.cpu().view(bits), kp.view(bits)), "append not bit-exact"
+    assert torch.equal(d.v_pool.cpu().view(bits), vp.view(bits)), "append not bit-exact"
     ref = oracle_paged.paged_prefill(wl.query, kp, vp, wl.block_tables, wl.context_lens, wl.cu_seqlens_q)
     truth = oracle_paged.paged_prefill(*_f64(wl.query, kp, vp), wl.block_tables, wl.context_lens, wl.cu_seqlens_q)
     # the first row of a chunk sees its prefix and itself
