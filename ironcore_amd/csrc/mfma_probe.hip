@@ -55,6 +55,9 @@ __global__ __launch_bounds__(4 * kWave) void mfma_probe_kernel(int iters, float 
                  : "v"(b));
 #undef IC_PROBE_STEP
     if ((it & 1023) == 1023) {  // keep the sums finite
+      // The compiler does not see the MFMAs inside the block above, so it cannot place the wait
+      // states a vector read of their results needs: wait out more than the longest MFMA first.
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3));
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         c0[i] *= 1e-3f;
@@ -64,6 +67,7 @@ __global__ __launch_bounds__(4 * kWave) void mfma_probe_kernel(int iters, float 
       }
     }
   }
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3));
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < 16; ++i) s += c0[i] + c1[i] + c2[i] + c3[i];
