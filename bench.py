@@ -192,11 +192,11 @@ def copy_calibration(torch, dev):
 def time_steps(torch, step, steps, warmup, event_launches=EVENT_LAUNCHES):
     """Run `warmup` untimed steps, then exactly `steps` timed ones bracketed by
     synchronisations (no events inside: an event costs a step a launch slot),
-    then a pass of `event_launches` further steps each of which records three
-    events: before the append, between the append and the dominant call, after
-    it.  `step(i, ev)` enqueues step i and records `ev[0..2]` when `ev` is not
+    then a pass of `event_launches` further steps each of which records an
+    event pair around its dominant call.  `step(i, ev)` enqueues step i and
+    records `ev[0]` before and `ev[1]` after the dominant call when `ev` is not
     None.  Returns (ms per step by wall clock, per-call ms of the dominant
-    call, per-call ms of the append before it)."""
+    call)."""
     for i in range(warmup):
         step(i, None)
     torch.cuda.synchronize()
@@ -205,16 +205,15 @@ def time_steps(torch, step, steps, warmup, event_launches=EVENT_LAUNCHES):
         step(i, None)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    dom, app = event_pass(torch, step, steps, event_launches)
-    return wall * 1e3 / steps, dom, app
+    return wall * 1e3 / steps, event_pass(torch, step, steps, event_launches)
 
 
 def event_pass(torch, step, first, n):
-    ev = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(3)) for _ in range(n)]
-    for i, trio in enumerate(ev):
-        step(first + i, trio)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for i, pair in enumerate(ev):
+        step(first + i, pair)
     torch.cuda.synchronize()
-    return [b.elapsed_time(c) for _, b, c in ev], [a.elapsed_time(b) for a, b, _ in ev]
+    return [a.elapsed_time(b) for a, b in ev]
 
 
 def after_idle(torch, step, idle_s, warmup, steps):
@@ -228,19 +227,18 @@ def after_idle(torch, step, idle_s, warmup, steps):
     torch.cuda.synchronize()
     time.sleep(idle_s)
     n = min(warmup + steps, 60)
-    dom, app = event_pass(torch, step, 0, n)
-    both = [d + a for d, a in zip(dom, app)]
-    window = both[warmup:] if warmup < n else both
-    return {"idle_s": round(idle_s, 2), "launches": n,
-            "dominant_call_ms": [round(x, 4) for x in dom], "append_ms": [round(x, 4) for x in app],
+    dom = event_pass(torch, step, 0, n)
+    window = dom[warmup:] if warmup < n else dom
+    return {"idle_s": round(idle_s, 2), "launches": n, "dominant_call_ms": [round(x, 4) for x in dom],
             "mean_of_timed_window_ms": round(sum(window) / len(window), 5),
-            "what": "append + dominant call by events for the first launches after the GPU sat idle as long as "
+            "what": "the dominant call by events for the first launches after the GPU sat idle as long as "
                     "during the parity gate's CPU oracle; the wall-timed steps start in the same state, and "
-                    "mean_of_timed_window_ms (launches warmup .. warmup+steps-1 of this pass) is what ms_per_step "
-                    "has to be compared with: after an idle gap the device runs its first millisecond of work "
-                    "at a high clock, then drops below its steady clock for a few milliseconds and recovers over "
-                    "tens of milliseconds, so a timed region of a few milliseconds right after the gate sits in "
-                    "that transient, while the steady-state event times behind `roofline` do not"}
+                    "mean_of_timed_window_ms (launches warmup .. warmup+steps-1 of this pass) is what the "
+                    "dominant call cost inside them: after an idle gap the device runs its first millisecond "
+                    "of work at a high clock, then drops below its steady clock for a few milliseconds and "
+                    "recovers over tens of milliseconds, so a timed region of a few milliseconds right after "
+                    "the gate sits in that transient, while the steady-state event times behind `roofline` "
+                    "do not"}
 
 
 def timed_oracle(fn, budget_s):
@@ -289,16 +287,14 @@ def bench_decode(args, torch, dev, workload):
 
     def step(i, ev):
         kp, vp = pools[i % len(pools)]
-        if ev:
-            ev[0].record()
         paged_ops.kv_append(k_new, v_new, kp, vp, slot_mapping)
         if ev:
-            ev[1].record()
+            ev[0].record()
         paged_ops.paged_decode(wl.query, kp, vp, wl.block_tables, wl.context_lens,
                                wl.max_context_len, out=out, min_chunk_tokens=args.min_chunk_tokens,
                                cohort_size=cohort, cohort_shared_blocks=shared)
         if ev:
-            ev[2].record()
+            ev[1].record()
 
     # parity gate on the tensors that are about to be timed: EVERY sequence of the batch against
     # the oracle, and the appended rows against the pool bit for bit
@@ -321,9 +317,16 @@ def bench_decode(args, torch, dev, workload):
     if args.copy_calibration:
         copy_calibration(torch, dev)
 
-    ms_per_step, decode_ms, append_ms = time_steps(torch, step, args.steps, args.warmup)
+    ms_per_step, decode_ms = time_steps(torch, step, args.steps, args.warmup)
     decode_ms_avg = sum(decode_ms) / len(decode_ms)
-    append_ms_avg = sum(append_ms) / len(append_ms)
+
+    def append_only(i, ev):
+        if ev:
+            ev[0].record()
+        paged_ops.kv_append(k_new, v_new, pools[0][0], pools[0][1], slot_mapping)
+        if ev:
+            ev[1].record()
+    append_ms_avg = statistics.mean(event_pass(torch, append_only, 0, 20))
     es = wl.query.element_size()
     decode_bytes = wl.algorithmic_bytes()
     append_bytes = 2 * (2 * b * gn * hd * es) + 8 * b
@@ -343,8 +346,9 @@ def bench_decode(args, torch, dev, workload):
                    "resident_layers": len(pools), "cohort_size": cohort,
                    "step": f"kv_append({b} rows) + paged_decode, one layer"},
         "parity_max_abs_vs_oracle": parity,
-        # wall time of a step beyond its two calls' steady-state event times (launch gaps, and whatever the
-        # device had not yet settled when the wall-timed steps ran)
+        # wall time of a step beyond its two calls' steady-state event times.  An event pair adds a few
+        # microseconds to what it brackets (for the 64-row append more than the 4.5 us the kernel takes by
+        # the profiler), so a step without launch gaps reads below zero here
         "append_ms": round(append_ms_avg, 5),
         "step_minus_kernels_ms": round(ms_per_step - decode_ms_avg - append_ms_avg, 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
@@ -380,15 +384,13 @@ def bench_prefill(args, torch, dev):
     out = torch.empty(wl.query.shape[0], wl.hn * wl.hd, dtype=wl.query.dtype, device=dev)
 
     def step(i, ev):
-        if ev:
-            ev[0].record()
         paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)
         if ev:
-            ev[1].record()
+            ev[0].record()
         paged_ops.paged_prefill(wl.query, wl.k_pool, wl.v_pool, wl.block_tables, wl.context_lens,
                                 wl.cu_seqlens_q, wl.max_chunk_len, causal=True, out=out)
         if ev:
-            ev[2].record()
+            ev[1].record()
 
     # parity gate: ALL sequences, all heads, against the oracle; the appended rows against the
     # pool bit for bit
@@ -410,9 +412,8 @@ def bench_prefill(args, torch, dev):
     if args.copy_calibration:
         copy_calibration(torch, dev)
 
-    ms_per_step, call_ms, app_in_step_ms = time_steps(torch, step, args.steps, args.warmup)
+    ms_per_step, call_ms = time_steps(torch, step, args.steps, args.warmup)
     call_avg = sum(call_ms) / len(call_ms)
-    app_in_step_avg = sum(app_in_step_ms) / len(app_in_step_ms)
     idle = after_idle(torch, step, min(max(cpu_s * cpu_runs, 0.5), 6.0), args.warmup, args.steps)
     flops = wl.flops()
     es = wl.query.element_size()
@@ -424,11 +425,11 @@ def bench_prefill(args, torch, dev):
     def append_only(i, ev):
         if ev:
             ev[0].record()
-            ev[1].record()
         paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)
         if ev:
-            ev[2].record()
-    _, app_ms, _ = time_steps(torch, append_only, 5, 5)
+            ev[1].record()
+    _, app_ms = time_steps(torch, append_only, 5, 5)
+    app_in_step_avg = statistics.mean(app_ms)
 
     # the same append with rotary embedding fused in (Q rotated in place, K rotated
     # into the pool, V copied), timed the same way on a scratch copy of the query
@@ -442,12 +443,11 @@ def bench_prefill(args, torch, dev):
     def rope_append_only(i, ev):
         if ev:
             ev[0].record()
-            ev[1].record()
         paged_ops.rope_kv_append(q_rot, wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping, pos,
                                  cos_t, sin_t)
         if ev:
-            ev[2].record()
-    _, rope_ms, _ = time_steps(torch, rope_append_only, 5, 5)
+            ev[1].record()
+    _, rope_ms = time_steps(torch, rope_append_only, 5, 5)
     rope_bytes = append_bytes + 2 * wl.query.numel() * es
     paged_ops.kv_append(wl.k_new, wl.v_new, wl.k_pool, wl.v_pool, wl.slot_mapping)  # leave the pool unrotated
 
