@@ -154,6 +154,9 @@ def parse():
                          "how much of the launch time is the clock the device holds under toggling operands)")
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="prefill: skip the 2 s measurement of the matrix rate the device sustains")
+    ap.add_argument("--no-after-idle", action="store_true",
+                    help="prefill: skip the pass that profiles the first launches after an idle gap (counter runs: "
+                         "its launches would enter the per-dispatch averages)")
     ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU baseline time budget per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -414,7 +417,8 @@ def bench_prefill(args, torch, dev):
 
     ms_per_step, call_ms = time_steps(torch, step, args.steps, args.warmup)
     call_avg = sum(call_ms) / len(call_ms)
-    idle = after_idle(torch, step, min(max(cpu_s * cpu_runs, 0.5), 6.0), args.warmup, args.steps)
+    idle = None if args.no_after_idle else after_idle(torch, step, min(max(cpu_s * cpu_runs, 0.5), 6.0),
+                                                      args.warmup, args.steps)
     flops = wl.flops()
     es = wl.query.element_size()
     append_bytes = 2 * 2 * wl.k_new.numel() * es
@@ -487,7 +491,7 @@ def bench_prefill(args, torch, dev):
         "parity_max_abs_vs_oracle": parity,
         "append_ms": round(app_in_step_avg, 5),
         "step_minus_kernels_ms": round(ms_per_step - call_avg - app_in_step_avg, 5),
-        "after_idle": idle,
+        **({"after_idle": idle} if idle is not None else {}),
         "append_hbm_gbps": round(append_bytes / (statistics.mean(app_ms) * 1e-3) / 1e9, 1),
         "rope_append_hbm_gbps": round(rope_bytes / (statistics.mean(rope_ms) * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,

@@ -231,12 +231,10 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int rsub = lane / CPR;  // row within the rows one load covers
   const char *stage_pool = side == 0 ? p.k_pool : p.v_pool;
   const int64_t head_off = (int64_t)kvh * p.stride_head;
-  // pool block of a row that starts a 16-row group (wave-uniform, scalar unit): a shift for
-  // power-of-two blocks, else a multiplication by the reciprocal the host prepared
-  auto block_of = [&](int row) {
-    return p.block_shift >= 0 ? row >> p.block_shift : (int)__umulhi((uint32_t)row >> 4, p.block_magic);
-  };
-  const int last_blk = SINGLE ? 0 : block_of((L - 1) & ~15);
+  // pool block of a row (wave-uniform: one multiplication on the scalar unit by the reciprocal
+  // of the block size the host prepared, whatever multiple of 16 the block size is)
+  auto block_of = [&](int row) { return (int)__umulhi((uint32_t)row, p.block_magic); };
+  const int last_blk = SINGLE ? 0 : block_of(L - 1);
   typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
   const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
   // byte offset, from the group's first row, of the chunk lane l fetches with load i: row
@@ -616,11 +614,12 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   for (int s = 0; s < 31; ++s)
     if ((1 << s) == a.pool.block_size) kp.block_shift = s;
   kp.block_magic = 0;
-  if (kp.block_shift < 0 && a.pool.block_size >= 16) {
-    // exact for token rows below 2^40 / block_size; longer tables are refused
-    kp.block_magic = (uint32_t)((1ull << 32) / (uint32_t)(a.pool.block_size / 16)) + 1u;
-    if (a.block_table_stride > 1 &&
-        a.block_table_stride * (int64_t)a.pool.block_size >= ((int64_t)1 << 40) / a.pool.block_size)
+  if (a.pool.block_size >= 2) {
+    kp.block_magic = (uint32_t)((1ull << 32) / (uint32_t)a.pool.block_size) + (kp.block_shift < 0 ? 1u : 0u);
+    // a block size that is no power of two: the reciprocal is exact for token rows below
+    // 2^32 / block_size; tables that reach further are refused
+    if (kp.block_shift < 0 && a.block_table_stride > 1 &&
+        a.block_table_stride * (int64_t)a.pool.block_size >= ((int64_t)1 << 32) / a.pool.block_size)
       return IC_ERR_UNSUPPORTED;
   }
   kp.group = a.hn / a.gn;

@@ -27,7 +27,8 @@ struct PrefillKP {
   int64_t num_blocks;
   int block_size;   // a multiple of 16 tokens
   int block_shift;  // log2(block_size) when it is a power of two, else -1
-  uint32_t block_magic;  // otherwise floor(2^32 / (block_size / 16)) + 1: n / (block_size / 16) == mulhi(n, magic)
+  uint32_t block_magic;  // row / block_size == mulhi(row, block_magic): 2^32 / block_size for a power of two
+                         // (exact for every row), else floor(2^32 / block_size) + 1 (exact below 2^32 / block_size)
   int group;        // query heads per KV head
   int gn;           // KV heads
   int n_units;      // n_seqs * gn
