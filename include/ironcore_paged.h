@@ -17,9 +17,22 @@
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *  - Return value: IC_OK (0) or a negative IC_ERR_* code.  Argument errors
  *    are detected on the host before anything is launched.  The library
- *    never throws, never exits the process and keeps no mutable global
- *    state, so calls may come from any host thread; ordering is the
- *    stream's.
+ *    never throws and never exits the process.  Calls may come from any
+ *    host thread; ordering is the stream's.  What the library remembers
+ *    between calls never shows in a result: per device, the CU count and
+ *    the address of the static scratch below; per process, the occupancy
+ *    the runtime reported for each decode kernel variant and LDS size
+ *    class (asked once, see ic_decode_occupancy_queries) and whether a
+ *    variant's dynamic-LDS limit has been raised.  All of it is written
+ *    once and read with atomics.
+ *  - Device memory the library owns: one array of IC_STATIC_SCRATCH_BYTES
+ *    (32 MiB), part of the code object, so every process that loads the
+ *    library holds it on each GPU it uses, whether or not it ever calls
+ *    ic_paged_decode_static (the only entry point that touches it).
+ *  - Head dimensions with attention kernels: 32, 64 and 128 (the append
+ *    entry points take any head dimension whose rows are a multiple of 16
+ *    bytes); others return IC_ERR_UNSUPPORTED.  Block sizes: any multiple
+ *    of 16 tokens.
  *  - Element type is selected by `dtype` (IC_DTYPE_*).  Strides are in
  *    ELEMENTS.  The head dimension is always contiguous.
  *
@@ -273,7 +286,9 @@ int ic_paged_decode_static(void *out, int64_t out_stride_seq,
  * j <= (L - C) + r.  Computes what attention.py:68-142 returns for
  * sq = C, sk = L with the causal mask of ironcore/language_model.py:109-114
  * shifted by the cached prefix.  With causal = 0 every query row sees all L
- * keys (the reference's attention_mask=None case).
+ * keys (the reference's attention_mask=None case).  bf16 / fp16 pools run on
+ * the 16-bit matrix-core kernel; fp32 pools on an fp32 kernel that keeps
+ * every product, sum and probability in fp32.
  *
  *   out           [n_tokens, hn*hd], row stride out_stride_token
  *   q             [n_tokens, hn, hd], row stride q_stride_token; the chunk of
@@ -308,7 +323,7 @@ int ic_paged_prefill(void *out, int64_t out_stride_token,
  * Hidden keys get the reference's FINITE fill value (attention.py:66): next to a
  * visible key they weigh nothing; a query row with no visible key returns the
  * plain average of V over its context, as the reference does.  A chunk may be
- * longer than its context here (sq > sk).  bf16 / fp16 only.
+ * longer than its context here (sq > sk).  bf16, fp16 and fp32.
  */
 int ic_paged_prefill_masked(void *out, int64_t out_stride_token,
                             const void *q, int64_t q_stride_token,
@@ -330,9 +345,9 @@ int ic_paged_prefill_masked(void *out, int64_t out_stride_token,
  * key_mask[i*key_mask_stride_seq + h*key_mask_stride_head + j] is nonzero
  * (key_mask_stride_head 0 = one mask row for all heads; key_mask_stride_seq
  * >= max_context_len).  Same finite-fill semantics as ic_paged_prefill_masked.
- * It is how an fp32 attention call with a general mask runs (one decode row
- * per query row; fp32 has no matrix-core path); 16-bit calls use
- * ic_paged_prefill_masked and get IC_ERR_UNSUPPORTED here.
+ * For single-token steps of an fp32 model under a general mask; chunks, and
+ * 16-bit calls of any length, use ic_paged_prefill_masked (16-bit pools get
+ * IC_ERR_UNSUPPORTED here).
  */
 int ic_paged_decode_masked(void *out, int64_t out_stride_seq,
                            const void *q, int64_t q_stride_seq,
