@@ -229,8 +229,13 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int grp = wave & 3;
   const int cc = lane % CPR;    // LDS slot (16-byte chunk of the row) this lane fills
   const int rsub = lane / CPR;  // row within the rows one load covers
-  const char *stage_pool = side == 0 ? p.k_pool : p.v_pool;
-  const int64_t head_off = (int64_t)kvh * p.stride_head;
+  // The address of a group is scalar work done once per tile in the vector step, whose length
+  // the launch time follows: 32-bit factors (the host refuses pool blocks of 4 GiB and more),
+  // one 32 x 32 -> 64-bit product per tile.
+  const char *pool_head = (side == 0 ? p.k_pool : p.v_pool) + (int64_t)kvh * p.stride_head * 2;
+  const uint32_t block_bytes = (uint32_t)(p.stride_block * 2);
+  const uint32_t token_bytes = (uint32_t)(p.stride_token * 2);
+  const int last_phys = (int)p.num_blocks - 1;
   // pool block of a row (wave-uniform: one multiplication on the scalar unit by the reciprocal
   // of the block size the host prepared, whatever multiple of 16 the block size is)
   auto block_of = [&](int row) { return (int)__umulhi((uint32_t)row, p.block_magic); };
@@ -238,32 +243,36 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   typedef const __attribute__((address_space(4))) int32_t *TablePtr;  // scalar (SMEM) loads
   const TablePtr table_row = (TablePtr)(unsigned long long)(p.block_tables + (int64_t)seq * p.bt_stride);
   // byte offset, from the group's first row, of the chunk lane l fetches with load i: row
-  // i*WR + rsub of the group, and the chunk whose place in that row is this lane's slot
+  // i*WR + rsub of the group, and the chunk whose place in that row is this lane's slot; less
+  // the 1 KiB per load that the load's instruction offset adds (see fetch_rows; rows are at
+  // least ROWB bytes apart, so this stays non-negative)
   uint32_t lane_src[NST];
 #pragma unroll
   for (int i = 0; i < NST; ++i) {
     const int r = i * WR + rsub;  // (a group starts at a multiple of 16 rows: r stands for the tile row)
     const int chunk = cc ^ (side == 0 ? swz_k(r) : swz_v(r));
-    lane_src[i] = (uint32_t)((int64_t)r * p.stride_token * 2 + chunk * 16);
+    lane_src[i] = (uint32_t)((int64_t)r * p.stride_token * 2 + chunk * 16) - i * WR * ROWB;
   }
   const uint32_t lds_pool = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)(side == 0 ? &s_k[0][0] : &s_v[0][0]);
   auto clamp_tile = [&](int tile) { return tile < n_tiles ? tile : n_tiles - 1; };
-  auto lookup = [&](int tile, int32_t &ent) {
+  // Table entry of this wave's group of `tile`, and the group's first row within its block.
+  auto lookup = [&](int tile, int32_t &ent, int &rem) {
     const int first = clamp_tile(tile) * kBN + 16 * grp;  // this wave's first row of the tile
     int blk = SINGLE ? 0 : block_of(first);
+    rem = first - blk * p.block_size;
     blk = blk < last_blk ? blk : last_blk;
     ent = table_row[blk];
   };
   // Issue the loads of this wave's group of `tile` into the tile's LDS buffer.
-  auto fetch_rows = [&](int tile, int32_t ent) {
-    const int first = clamp_tile(tile) * kBN + 16 * grp;
-    int64_t phys = ent;
+  auto fetch_rows = [&](int tile, int32_t ent, int rem) {
+    int phys = ent;
     // A corrupt table entry must not become an out-of-pool address.
     phys = phys < 0 ? 0 : phys;
-    phys = phys >= p.num_blocks ? p.num_blocks - 1 : phys;
+    phys = phys > last_phys ? last_phys : phys;
     const uint32_t dst = lds_pool + (uint32_t)((tile & (NB - 1)) * (kBN * ROWB) + 16 * grp * ROWB);
     if (SINGLE) {
-      const char *base = stage_pool + (phys * p.stride_block + head_off) * 2;
+      const int first = clamp_tile(tile) * kBN + 16 * grp;
+      const char *base = pool_head + (uint64_t)(uint32_t)phys * block_bytes;
 #pragma unroll
       for (int i = 0; i < NST; ++i) {
         int row = first + rsub + i * WR;
@@ -274,12 +283,15 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
                      :: "s"(dst + i * WR * ROWB), "v"(src) : "memory", "m0");
       }
     } else {
-      const int rem = first - block_of(first) * p.block_size;
-      const char *base = stage_pool + (phys * p.stride_block + head_off + (int64_t)rem * p.stride_token) * 2;
+      const char *base = pool_head + ((uint64_t)(uint32_t)phys * block_bytes + (uint32_t)rem * token_bytes);
+      // One LDS base for the group's loads: a load's instruction offset moves its LDS address
+      // AND its memory address, here by the 1 KiB that one load fills (lane_src takes it off the
+      // memory side again).
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" :: "s"(dst) : "memory", "m0");
 #pragma unroll
       for (int i = 0; i < NST; ++i)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst + i * WR * ROWB), "v"(lane_src[i]), "s"(base) : "memory", "m0");
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2"
+                     :: "v"(lane_src[i]), "s"(base), "n"(i * WR * ROWB) : "memory", "m0");
     }
   };
   // The loads of `tile` have arrived (everything but the `younger` loads issued after them); rows
@@ -293,7 +305,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
       asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NST) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NST) : "memory");
-    if (side == 1 && tile < n_tiles && tile * kBN + 16 * grp + 16 > L) {
+    if (tile == n_tiles - 1 && side == 1 && tile * kBN + 16 * grp + 16 > L) {  // (only a sweep's last tile can reach past L)
       char *buf = s_v[tile & (NB - 1)] + 16 * grp * ROWB + lane * 16;
       const int row = tile * kBN + 16 * grp + rsub;
 #pragma unroll
@@ -309,6 +321,9 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   const int vq = (lane & 15) >> 2;
   const int v_lane = (4 * hh + vq) * ROWB + ((swz_v(vq) >> 2) << 6) + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
 
+  // First tile that needs the mask: the one the causal diagonal of the wave's first row enters
+  // (tile*64 + 63 > P + that row), or without the causal rule a last tile the context does not fill.
+  const int mask_from = __builtin_amdgcn_readfirstlane(causal ? (P + q0 + wave * 32 + 1) / kBN : L / kBN);
   f32x16_t s[TB];        // S^T of the tile in flight: (token, query n)
   Vec16 pb[kBN / 16];    // its probabilities as MFMA B operands
 
@@ -346,7 +361,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   auto softmax = [&](int tile) {
     // s[tb][i] is (token tile*64 + tb*32 + 4*hh + 8*(i/4) + i%4, query n)
     const int tok_base = tile * kBN + 4 * hh;
-    const bool need_mask = causal ? (tile * kBN + kBN - 1 > P + q0 + wave * 32) : (tile * kBN + kBN > L);
+    const bool need_mask = tile >= mask_from;
     if (need_mask) {  // tiles that touch the causal diagonal (or the context end)
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
@@ -463,6 +478,7 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // 2k-1 for K, 2k+1 for V: one barrier before the issue at the latest).  So a tile's loads are
   // in flight for four phases, and a wave always has two tiles of its pool on the way.
   int32_t ent;  // table entry of the tile the next vector step fetches
+  int ent_rem;  // and the first row of this wave's group within that block
   auto matrix_step = [&](int k) {
     // the wave in its matrix step goes first when both waves of the SIMD have an instruction ready:
     // an MFMA or operand read issued late idles the matrix pipe, a softmax instruction issued late
@@ -484,8 +500,8 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   auto vector_step = [&](int j, int tile) {
     __builtin_amdgcn_s_setprio(0);
     landed(tile, 1);
-    fetch_rows(tile + 2, ent);
-    lookup(tile + 3, ent);  // for the next vector step, which fetches tile + 3
+    fetch_rows(tile + 2, ent, ent_rem);
+    lookup(tile + 3, ent, ent_rem);  // for the next vector step, which fetches tile + 3
     if (j >= 0 && j < my_tiles) {
       softmax(j);
     } else {
@@ -497,21 +513,23 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_prefill_kernel(const Pr
   // (all table entries first, then all tiles: one round trip each, not one per tile)
   if (side == 0) {
     int32_t e0, e1, e2;
-    lookup(0, e0);
-    lookup(1, e1);
-    lookup(2, e2);
-    lookup(3, ent);  // the first vector step waits for K(1) and fetches K(3)
-    fetch_rows(0, e0);
-    fetch_rows(1, e1);
-    fetch_rows(2, e2);
+    int r0, r1, r2;
+    lookup(0, e0, r0);
+    lookup(1, e1, r1);
+    lookup(2, e2, r2);
+    lookup(3, ent, ent_rem);  // the first vector step waits for K(1) and fetches K(3)
+    fetch_rows(0, e0, r0);
+    fetch_rows(1, e1, r1);
+    fetch_rows(2, e2, r2);
     landed(0, 2);
   } else {
     int32_t e0, e1;
-    lookup(0, e0);
-    lookup(1, e1);
-    lookup(2, ent);  // the first vector step waits for V(0) and fetches V(2)
-    fetch_rows(0, e0);
-    fetch_rows(1, e1);
+    int r0, r1;
+    lookup(0, e0, r0);
+    lookup(1, e1, r1);
+    lookup(2, ent, ent_rem);  // the first vector step waits for V(0) and fetches V(2)
+    fetch_rows(0, e0, r0);
+    fetch_rows(1, e1, r1);
   }
   __syncthreads();
   // Both sides pass the same number of barriers.
@@ -635,6 +653,15 @@ int launch_paged_prefill(const PrefillArgs &a, hipStream_t stream) {
   kp.mask_keys = a.mask_keys > 0x7fffffff ? 0x7fffffff : (int)a.mask_keys;
   if ((int64_t)a.max_chunk_len >= (int64_t)65535 * 128 || a.hn > 65535 || a.n_seqs > 65535)
     return IC_ERR_UNSUPPORTED;
+  // The 16-bit kernel addresses a block with 32-bit byte offsets (a block, and in a block table's
+  // blocks the rows from a block's start to any of its 16-row groups, stay below 4 GiB; the 16
+  // rows of a group below 4 GiB in any case) and numbers blocks with 32 bits, as the tables do.
+  if (a.dtype != IC_DTYPE_F32) {
+    const int64_t span_rows = a.block_table_stride > 1 && a.pool.block_size > 16 ? a.pool.block_size : 16;
+    if (a.pool.stride_block >= ((int64_t)1 << 31) || a.pool.stride_token * span_rows >= ((int64_t)1 << 31) ||
+        a.pool.num_blocks > 0x7fffffff)
+      return IC_ERR_UNSUPPORTED;
+  }
   switch (a.dtype) {
     case IC_DTYPE_BF16: return launch_mode<MmaBf16>(kp, a, stream);
     case IC_DTYPE_F16: return launch_mode<MmaF16>(kp, a, stream);

@@ -104,15 +104,18 @@ def test_prefill_argument_errors():
     lib = _lib.load()
 
     def call(out=1 << 12, q=1 << 13, kp=1 << 14, vp=1 << 15, bt=1 << 16, cl=1 << 17, cu=1 << 18,
-             n=4, chunk=512, hn=32, gn=32, hd=128, dtype=0, qs=4096):
-        return lib.ic_paged_prefill(out, 4096, q, qs, kp, vp, 65536, 2048, 128, bt, 300, cl, cu, n, chunk,
-                                    hn, gn, hd, 16, 1000, 0.0884, 1, dtype, None)
+             n=4, chunk=512, hn=32, gn=32, hd=128, dtype=0, qs=4096, sb=65536, st=128, bs=16):
+        return lib.ic_paged_prefill(out, 4096, q, qs, kp, vp, sb, 2048, st, bt, 300, cl, cu, n, chunk,
+                                    hn, gn, hd, bs, 1000, 0.0884, 1, dtype, None)
     assert call(n=0, q=None) == 0
     assert call(cu=None) == -1
     assert call(hn=33) == -2
     assert call(qs=100) == -2
     assert call(dtype=5) == -3
     assert call(q=(1 << 13) + 8) == -6
+    # the 16-bit kernel addresses inside a pool block with 32 bits: blocks of 4 GiB and more are refused
+    assert call(sb=1 << 31) == -3
+    assert call(st=1 << 24, bs=128) == -3
 
 
 def test_masked_entry_points_argument_errors():
