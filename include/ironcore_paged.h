@@ -295,6 +295,9 @@ int ic_paged_decode_static(void *out, int64_t out_stride_seq,
  *                 sequence i is rows cu_seqlens_q[i] .. cu_seqlens_q[i+1]-1
  *   cu_seqlens_q  int32 [n_seqs + 1]
  *   max_chunk_len upper bound on any chunk length (sizes the grid)
+ * The 16-bit kernel addresses inside a pool block with 32 bits: a call whose
+ * pool_stride_block, or pool_stride_token times the rows of a block, reaches
+ * 2^31 elements (a block of 4 GiB) returns IC_ERR_UNSUPPORTED.
  */
 int ic_paged_prefill(void *out, int64_t out_stride_token,
                      const void *q, int64_t q_stride_token,
