@@ -21,8 +21,11 @@ runs on the same chunked-prefill kernel by viewing ``key``/``value`` as a pool
 with one block per sequence.  bf16 and fp16 tensors take the 16-bit matrix-core
 kernels, fp32 tensors (what the reference's own contract tests pass,
 tests/test_attention.py:143-161) the fp32 ones, with every product, sum and
-probability in fp32.  Every path runs the hand-written HIP kernels; there is
-no torch fallback.
+probability in fp32.  The reference's second branch is kept as well: when
+``config.trainer.use_flash_attn`` is set and the flash-attn import worked, the
+dense call goes through ``_flash_attention`` (causal, the mask ignored,
+attention.py:230-250), here on the same kernels.  Every path runs the
+hand-written HIP kernels; there is no torch fallback.
 """
 from __future__ import annotations
 
@@ -36,6 +39,14 @@ from torch import nn
 
 from .. import paged_ops
 from .module import BaseModule, get_model_dtype
+
+# The reference takes its flash branch only when this import worked
+# (ironcore/layers/attention.py:14-17,230).  Here the name is nothing but that
+# switch: the branch runs on the kernels of this package, never on the wheel.
+try:
+    from flash_attn import flash_attn_varlen_func
+except ImportError:
+    flash_attn_varlen_func = None
 
 
 # attention_mask tensor -> what _classify_mask found for it: id -> (weak reference, (version, shapes), kind, bytes).
@@ -189,13 +200,47 @@ class Attention(BaseModule):
         if rotary_pos_emb is not None:
             raise ValueError("without a KV cache, rotate query and key before the call "
                              "(ironcore/models/transformer.py:95-98)")
+        if self.config.trainer.use_flash_attn and flash_attn_varlen_func is not None:
+            # the reference's flash branch: causal, the mask ignored (attention.py:230,240-250)
+            sq, sk = query.size(1), key.size(1)
+            return self._flash_attention(query, key, value, sq, sk, sq, sk, causal=True, window_size=(-1, -1))
         return self._dense(query, key, value, attention_mask)
+
+    def _flash_attention(self, query, key, value, seq_len_q, seq_len_kv, max_seqlen_q, max_seqlen_k,
+                         causal=False, window_size=(-1, -1), alibi_slopes=None):
+        """The reference's flash branch (attention.py:144-206) on this package's
+        kernels: every sequence whole (the reference builds equal-length
+        cu_seqlens, attention.py:170-183), ``causal`` aligned to the bottom
+        right as flash-attn aligns it (row i sees keys j <= (sk - sq) + i; a row
+        that sees no key returns zeros), which for sq == sk is the mask the
+        reference's own tests set beside it (tests/test_attention.py:618-671).
+        KV heads follow the GQA map of the dense branch, as those tests expect
+        (:673-730).  Sliding windows, ALiBi slopes and attention dropout (which
+        the wheel applies whatever the module's mode) are not built."""
+        if tuple(window_size) != (-1, -1) or alibi_slopes is not None:
+            raise NotImplementedError("sliding-window and ALiBi attention are not built")
+        if self.config.model.dropout_attn > 0.0:
+            raise NotImplementedError("the flash branch applies dropout_attn in every mode; the kernels "
+                                      "implement dropout_attn == 0")
+        b, sq, hn, hd = query.shape
+        sk = key.shape[1]
+        if (seq_len_q, seq_len_kv) != (sq, sk):
+            raise ValueError(f"seq_len_q / seq_len_kv {seq_len_q} / {seq_len_kv} do not match the tensors ({sq} / {sk})")
+        if not causal or sq <= sk:
+            return self._attend_dense(query, key, value, bool(causal), None)
+        out = query.new_zeros(b, sq, hn * hd)   # rows above the bottom-right triangle see no key
+        if sk > 0:
+            out[:, sq - sk:] = self._attend_dense(query[:, sq - sk:], key, value, True, None)
+        return out
 
     def _dense(self, query, key, value, attention_mask):
         b, sq, hn, hd = query.shape
-        sk, gn = key.shape[1], key.shape[2]
+        sk = key.shape[1]
         kind, mask = self._classify_mask(attention_mask, b, sq, sk, hn)
-        causal = kind == "causal"
+        return self._attend_dense(query, key, value, kind == "causal", mask)
+
+    def _attend_dense(self, query, key, value, causal, mask):
+        b, sq, hn, hd = query.shape
         if hd not in paged_ops.SUPPORTED_HEAD_DIMS:
             # The reference takes any d_model // heads (attention.py:51).  Zero columns appended
             # to query, key and value change no score (the scale stays 1/sqrt(hd)) and add zero

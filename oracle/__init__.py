@@ -51,5 +51,9 @@ Committed vectors                 tests/golden/*.npz (float64-loop attention
                                   weights), checked by tests/test_golden.py.
 _flash_attention numerics         parity unpinned (third-party flash_attn wheel,
                                   absent here; ironcore/layers/attention.py:
-                                  144-206).  Not restated.
+                                  144-206).  Not restated: the layer's flash
+                                  branch is checked against dense_attention
+                                  under the causal mask, the comparison the
+                                  reference's own tests make
+                                  (tests/test_attention.py:618-789).
 """
