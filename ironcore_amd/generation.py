@@ -22,7 +22,6 @@ layers/rotary.py).
 """
 from __future__ import annotations
 
-import math
 from typing import Optional, Sequence
 
 import torch
@@ -264,20 +263,10 @@ class LanguageModel(BaseModule):
         self.init_weights()
 
     def init_weights(self):
-        """ironcore/layers/module.py:43-76 at tensor-parallel size 1: biases 0,
-        norm scales 1, everything else N(0, init_std), residual projections
-        N(0, init_std / sqrt(2 * layers)); padded vocabulary rows zeroed."""
-        std = self.init_std
+        """The layers' initialisation (ironcore/layers/module.py:43-76), then the
+        padded vocabulary rows zeroed."""
+        super().init_weights()
         with torch.no_grad():
-            for name, param in self.named_parameters():
-                if "bias" in name:
-                    param.zero_()
-                elif "norm" in name:
-                    param.fill_(1.0)
-                elif name.endswith("output.weight") or name.endswith("down_proj.weight"):
-                    param.normal_(mean=0.0, std=std / math.sqrt(2 * self.config.model.num_layers))
-                else:
-                    param.normal_(mean=0.0, std=std)
             self.embedding.word_embeddings.weight[self.vocab_size:].zero_()
 
     def forward(self, input_ids, labels=None, *, kv_cache: Optional[PagedKVCache] = None,
