@@ -116,6 +116,14 @@ def test_random_prefill_head_dim_32(gpu, case):
     _random_prefill(gpu, 6000 + case, np.random.default_rng(6000 + case), dims=(32,))
 
 
+@pytest.mark.parametrize("case", range(24))
+def test_random_prefill_block_sizes_beyond_powers_of_two(gpu, case):
+    """16-bit pools whose blocks are multiples of 16 that are no power of two (the block of a row
+    by the reciprocal multiplication, groups that start inside a block), all three head dims."""
+    _random_prefill(gpu, 8000 + case, np.random.default_rng(8000 + case), dims=(32, 64, 128),
+                    blocks=(48, 80, 96, 112, 144, 176))
+
+
 @pytest.mark.parametrize("case", range(32))
 def test_random_prefill_fp32(gpu, case):
     """fp32 pools (the fp32 matrix-instruction kernel), all three head dims, block sizes that are no
